@@ -553,6 +553,49 @@ int ll_sample_top_p(int64_t* out, const void* logits, const float* temperature, 
                     const float* uniform, const void* greedy, int64_t batch, int64_t vocab,
                     int64_t stride, int dtype, void* stream);
 
+/* ---- ragged steps with a 32-bit residual stream (csrc/seq_mix.hip, csrc/ragged_attn.hip) -----------------------------
+ * A step carries b sequences; sequence i brings tokens seq_start[i] .. seq_start[i + 1] - 1 of the flat token arrays, the
+ * first of them at position seq_first_pos[i] of the sequence (0: the sequence starts here and has no state yet), with its
+ * fixed-size state in slot seq_slot[i]; tok_seq[t] / tok_pos[t] name a token's sequence and position.  dtype = storage type
+ * of activations and weights (LL_F16 / LL_BF16 / LL_F32); residual stream, norms, recurrent state, attention scores: fp32.
+ *
+ * ll_add_rmsnorm_shift: s = x_in + delta (delta may be NULL; else s is written to x_out), h = s / sqrt(mean(s^2) + eps) * w,
+ * y = h + (h_prev - h) * shift (shift may be NULL: y = h), h_prev = h of the sequence's previous token (zeros at position
+ * 0; from the state slot at the start of a run).  state = [2][state_half] floats, half seq_parity[i] is read and the other
+ * half written (h of the run's last token, at slot * width).  x_out must differ from x_in when delta and shift are given. */
+int ll_add_rmsnorm_shift(const float* x_in, const void* delta, float* x_out, const void* weight, const void* shift,
+                         void* y, int64_t n, int64_t width, float eps, const int32_t* tok_seq,
+                         const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot,
+                         const int32_t* seq_parity, float* state, int64_t state_half, int dtype, void* stream);
+/* xIELU with pq = (p, q): z > 0: softplus(p) z^2 + z / 2;  else (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2. */
+int ll_xielu(void* y, const void* z, const void* pq, int64_t n, int dtype, void* stream);
+/* out [n, 2 width] = [a + a_delta | b] cast to dtype (a_delta in dtype, or NULL);  x [n, width] (fp32) = y + bias (bias
+ * [width] or NULL). */
+int ll_cast_pair(void* out, const float* a, const void* a_delta, const float* b, int64_t n, int64_t width, int dtype,
+                 void* stream);
+int ll_residual_set(float* x, const void* y, const void* bias, int64_t n, int64_t width, int dtype, void* stream);
+/* Gated linear recurrence per (sequence, head): f = lower + (1 - lower) sigmoid(f_raw + f_bias), S <- diag(f) S + (1 - f) v^T,
+ * o = S^T silu(q_raw), out = o / sqrt(mean_dv(o^2) + eps) * norm_w.  q, f [n, >= heads dk], v [n, >= heads dv] share the
+ * row stride ld; state [slots][heads][dk][dv] fp32 (read when seq_first_pos > 0, written at the end of the run). */
+int ll_gated_linear_scan_supported(int64_t dk, int64_t dv);
+int ll_gated_linear_scan(const void* q, const void* f, const void* v, int64_t ld, const void* f_bias, const void* lower,
+                         const void* norm_w, float eps, void* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
+                         const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, float* state,
+                         int dtype, void* stream);
+/* Rows [q (heads dk) | k (kv_heads dk) | v (kv_heads dv)] of stride ld: q and k RMS-normed per head (weights [dk] or NULL),
+ * q times 1 + temp_coef ln(floor((pos + 1) / temp_every) + 1); q -> q_out [n, heads, dk]; k, v -> cache rows select[t] of
+ * k_cache [rows, kv_heads, dk] / v_cache [rows, kv_heads, dv]. */
+int ll_qk_norm_cache(const void* qkv, int64_t ld, const void* q_w, const void* k_w, float eps, float temp_coef,
+                     int64_t temp_every, const int32_t* tok_pos, const int32_t* select, void* q_out, void* k_cache,
+                     void* v_cache, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int dtype,
+                     void* stream);
+/* Causal softmax attention of every token against positions 0 .. tok_pos[t] of its sequence (cache rows through
+ * token_table[seq_req[tok_seq[t]]][pos]); score = (q . k) scale; sink [heads] or NULL adds exp(sink_h) to the denominator. */
+int ll_ragged_attention(const void* q, const void* k_cache, const void* v_cache, const int32_t* token_table,
+                        int64_t tt_stride, const int32_t* seq_req, const int32_t* tok_seq, const int32_t* tok_pos,
+                        const void* sink, float scale, void* out, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk,
+                        int64_t dv, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -14,6 +14,9 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("LL_LIB_OVERRIDE") or os.path.join(_HERE, "lib", "liblite_llama_amd.so")  # override: A/B builds
+# A PART library (build.py::PARTS) holds the sources one model family needs: a fresh checkout that serves only that family
+# compiles those and nothing else.  The full library, when it is there, serves everybody.
+PART_PATH = os.path.join(_HERE, "lib", "liblite_llama_amd_{part}.so")
 
 LL_F16, LL_BF16, LL_F32 = 0, 1, 2
 LL_I32, LL_I64 = 0, 1
@@ -107,6 +110,14 @@ SIGNATURES = {
     "ll_repetition_penalty": [P, P, P, P, P, F, L, L, L, L, L, L, L, I, I, P],
     "ll_sample_top_p": [P, P, P, P, P, P, L, L, L, I, P],
     "ll_argmax_split": [P, P, L, L, L, I, P, I, P],
+    "ll_add_rmsnorm_shift": [P, P, P, P, P, P, L, L, F, P, P, P, P, P, P, L, I, P],
+    "ll_xielu": [P, P, P, L, I, P],
+    "ll_cast_pair": [P, P, P, P, L, L, I, P],
+    "ll_residual_set": [P, P, P, L, L, I, P],
+    "ll_gated_linear_scan_supported": [L, L],
+    "ll_gated_linear_scan": [P, P, P, L, P, P, P, F, P, L, L, L, L, P, P, P, P, I, P],
+    "ll_qk_norm_cache": [P, L, P, P, F, F, L, P, P, P, P, P, L, L, L, L, L, I, P],
+    "ll_ragged_attention": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, L, I, P],
 }
 
 _RETURNS_I64 = {"ll_kv_alloc_scratch_bytes", "ll_tp_oneshot_flag_words", "ll_moe_router_workspace_floats", "ll_moe_align_workspace_ints"}
@@ -117,18 +128,35 @@ class KernelError(RuntimeError):
     """A C-ABI entry point returned a negative status."""
 
 
+_part = None  # name of the part library to fall back to when the full library is not built
+
+
+def use_part(name: str) -> None:
+    """Let :func:`lib` serve a process that only needs the part library ``name``: the full library is loaded when it is built
+    and current, else the part is compiled if need be (build.py::ensure) and loaded (entry points of other sources are then
+    simply not there: touching one raises ``AttributeError``)."""
+    global _part
+    _part = name
+
+
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
+        path, partial = LIB_PATH, bool(os.environ.get("LL_LIB_OVERRIDE"))
+        if _part is not None and not partial:
+            from . import build
+
+            path = build.ensure(_part)
+            partial = path != LIB_PATH
+        if not os.path.exists(path):
             raise RuntimeError(
                 f"lite_llama_amd: HIP library not found at {LIB_PATH}; run "
                 "`python -m lite_llama_amd.build` (there is no CPU/eager fallback)"
             )
-        handle = ctypes.CDLL(LIB_PATH)
+        handle = ctypes.CDLL(path)
         for name, argtypes in SIGNATURES.items():
-            if os.environ.get("LL_LIB_OVERRIDE") and not hasattr(handle, name):
-                continue  # A/B builds of an older source (benchmarks only): a call to the missing entry still fails loudly
+            if partial and not hasattr(handle, name):
+                continue  # A/B builds of an older source, part libraries: a call to the missing entry still fails loudly
             fn = getattr(handle, name)  # AttributeError if the symbol is missing -> loud
             fn.argtypes = argtypes
             fn.restype = ctypes.c_int64 if name in _RETURNS_I64 else c_int
@@ -136,6 +164,11 @@ def lib() -> ctypes.CDLL:
             raise RuntimeError("lite_llama_amd: ABI version mismatch between _lib.py and the .so")
         _lib = handle
     return _lib
+
+
+def has(name: str) -> bool:
+    """Whether the loaded library exports ``name`` (a part library holds only its own sources' entries)."""
+    return hasattr(lib(), name)
 
 
 def stream_ptr() -> int:

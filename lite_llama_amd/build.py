@@ -20,11 +20,17 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "liblite_llama_amd.so"
 ARCH = "gfx950"
-FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off"]
+FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off",
+         # no packed fp32 arithmetic from ordinary float code (the host pass warns that it does not know the feature)
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 FLAGS += os.environ.get("LL_EXTRA_HIPCC_FLAGS", "").split()  # debug builds (e.g. -DV2_DEBUG_ABLATE)
 # per-source flags.  gemm_short.hip: its kernel's first 16 argument dwords arrive in SGPRs with the wave (gfx950 kernarg preload)
 # instead of through dependent scalar loads -- a launch of ~5 us spends ~0.3 us there otherwise.
 FILE_FLAGS = {"gemm_short.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"]}
+
+
+# part libraries: the sources ONE model family needs (a fresh checkout serving only that family builds nothing else)
+PARTS = {"ragged": ["seq_mix.hip", "ragged_attn.hip", "kv_paged.hip", "kv_ops.hip", "sampler.hip"]}
 
 
 def flags_for(src: str) -> list[str]:
@@ -57,14 +63,28 @@ def lib_path() -> str:
     return os.path.join(LIBDIR, LIBNAME)
 
 
-def build(force: bool = False, verbose: bool = True) -> str:
-    os.makedirs(LIBDIR, exist_ok=True)
-    srcs = sources()
+def part_path(part: str) -> str:
+    return os.path.join(LIBDIR, f"liblite_llama_amd_{part}.so")
+
+
+def ensure(part: str, verbose: bool = False) -> str:
+    """What a model family's entry point calls first: the full library if it is built and current, else the family's part
+    library, compiled now if it is missing or stale."""
     stamp = os.path.join(LIBDIR, "build.stamp")
+    if os.path.exists(lib_path()) and os.path.exists(stamp) and open(stamp).read().strip() == _digest(sources()):
+        return lib_path()
+    return build(verbose=verbose, part=part)
+
+
+def build(force: bool = False, verbose: bool = True, part: str | None = None) -> str:
+    os.makedirs(LIBDIR, exist_ok=True)
+    srcs = sources() if part is None else [os.path.join(CSRC, f) for f in PARTS[part]]
+    target = lib_path() if part is None else part_path(part)
+    stamp = os.path.join(LIBDIR, "build.stamp" if part is None else f"build_{part}.stamp")
     digest = _digest(srcs)
-    if not force and os.path.exists(lib_path()) and os.path.exists(stamp):
+    if not force and os.path.exists(target) and os.path.exists(stamp):
         if open(stamp).read().strip() == digest:
-            return lib_path()
+            return target
     hipcc = _hipcc()
     objdir = os.path.join(LIBDIR, "obj")
     os.makedirs(objdir, exist_ok=True)
@@ -74,18 +94,21 @@ def build(force: bool = False, verbose: bool = True) -> str:
         cmd = [hipcc, *flags_for(src), "-c", src, "-o", obj]
         if verbose:
             print("[build]", " ".join(cmd), flush=True)
-        subprocess.run(cmd, check=True)
+        done = subprocess.run(cmd, stderr=None if verbose else subprocess.PIPE, text=True)
+        if done.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{done.stderr or ''}")
         return obj
 
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         objs = list(ex.map(compile_one, srcs))
-    cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", lib_path()]
+    cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", target + ".tmp"]
     if verbose:
         print("[build]", " ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
+    os.replace(target + ".tmp", target)
     with open(stamp, "w") as f:
         f.write(digest)
-    return lib_path()
+    return target
 
 
 if __name__ == "__main__":

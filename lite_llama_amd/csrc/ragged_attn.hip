@@ -1,0 +1,220 @@
+// Softmax attention over RAGGED steps against a paged cache, for head geometries the rotary llama kernels do not cover:
+// separate key and value widths, per-head RMS norm of queries and keys, a position-dependent query temperature instead of a
+// rotation, and a learned per-head SINK in the softmax denominator.
+//
+//   ll_qk_norm_cache     fused projection rows [q | k | v] -> normed, temperature-scaled queries; normed keys and raw values
+//                        written to the cache rows of their tokens
+//   ll_ragged_attention  every token of the step against keys 0 .. its own position of its sequence, read through the
+//                        per-token row table; scores, softmax and the running output in fp32
+//
+// The sink is a virtual key with score sink_h (not scaled) and a zero value: the running softmax simply STARTS at
+// (max = sink, sum = 1, output = 0).  A token's result depends only on its own position and on the cache rows of its
+// sequence, visited in a fixed order: how a prompt was cut into steps, or what else rides in the step, cannot change it.
+#include "common.h"
+
+namespace {
+
+template <int DT>
+__device__ __forceinline__ float ldv(const void* p, int64_t i) {
+  if constexpr (DT == LL_F32) return ((const float*)p)[i];
+  else return to_f32<DT>(((const uint16_t*)p)[i]);
+}
+template <int DT>
+__device__ __forceinline__ void stv(void* p, int64_t i, float v) {
+  if constexpr (DT == LL_F32) ((float*)p)[i] = v;
+  else ((uint16_t*)p)[i] = from_f32<DT>(v);
+}
+
+// One wave per (token, item): items 0 .. H - 1 = query heads, H .. H + G - 1 = key heads, then G value heads.
+template <int DT>
+__global__ __launch_bounds__(256) void qk_norm_cache_kernel(
+    const void* __restrict__ qkv, int64_t ld, const void* __restrict__ q_w, const void* __restrict__ k_w, float eps,
+    float temp_coef, int temp_every, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ select,
+    void* __restrict__ q_out, void* __restrict__ k_cache, void* __restrict__ v_cache, int64_t n, int heads, int kv_heads, int dk,
+    int dv) {
+  const int items = heads + 2 * kv_heads;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (w >= n * items) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = w / items;
+  const int item = (int)(w - t * items);
+  const int64_t row = select[t];
+  if (item >= heads + kv_heads) {  // value head: copy
+    const int gidx = item - heads - kv_heads;
+    const int64_t src = t * ld + (int64_t)(heads + kv_heads) * dk + (int64_t)gidx * dv;
+    for (int c = lane; c < dv; c += 64) stv<DT>(v_cache, (row * kv_heads + gidx) * dv + c, ldv<DT>(qkv, src + c));
+    return;
+  }
+  const bool is_q = item < heads;
+  const int64_t src = t * ld + (int64_t)item * dk;
+  float ss = 0.f;
+  for (int c = lane; c < dk; c += 64) {
+    const float x = ldv<DT>(qkv, src + c);
+    ss += x * x;
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)dk + eps);
+  float temp = 1.0f;
+  if (is_q && temp_coef != 0.f) temp = 1.0f + temp_coef * logf((float)((tok_pos[t] + 1) / temp_every) + 1.0f);
+  const void* wt = is_q ? q_w : k_w;
+  for (int c = lane; c < dk; c += 64) {
+    float r = ldv<DT>(qkv, src + c) * inv;
+    if (wt) r *= ldv<DT>(wt, c);
+    if (is_q) stv<DT>(q_out, (t * heads + item) * dk + c, r * temp);
+    else stv<DT>(k_cache, (row * kv_heads + (item - heads)) * dk + c, r);
+  }
+}
+
+// dot of an fp32 LDS vector with a contiguous cache row, channels in order; 16-byte loads when the row allows them
+template <int DT>
+__device__ __forceinline__ float dot_row(const float* __restrict__ a, const void* __restrict__ rowp, int64_t at, int dk, bool vec) {
+  float d = 0.f;
+  if constexpr (DT == LL_F32) {
+    const float* r = (const float*)rowp + at;
+    if (vec) {
+      for (int c = 0; c < dk; c += 4) {
+        const f32x4 x = *reinterpret_cast<const f32x4*>(r + c);
+        d += a[c] * x[0]; d += a[c + 1] * x[1]; d += a[c + 2] * x[2]; d += a[c + 3] * x[3];
+      }
+    } else {
+      for (int c = 0; c < dk; ++c) d += a[c] * r[c];
+    }
+  } else {
+    const uint16_t* r = (const uint16_t*)rowp + at;
+    if (vec) {
+      for (int c = 0; c < dk; c += 8) {
+        const U16x8 x = *reinterpret_cast<const U16x8*>(r + c);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d += a[c + i] * to_f32<DT>(x.v[i]);
+      }
+    } else {
+      for (int c = 0; c < dk; ++c) d += a[c] * to_f32<DT>(r[c]);
+    }
+  }
+  return d;
+}
+
+// One wave per (token, query head).  Keys in tiles of 64: lane j scores key base + j (a contiguous dk-row of the cache),
+// the tile's weights go through LDS, then lane c accumulates channel c (and c + 64, ...) of the output over the tile.
+template <int DT, int VPL>
+__global__ __launch_bounds__(256) void ragged_attention_kernel(
+    const void* __restrict__ q, const void* __restrict__ k_cache, const void* __restrict__ v_cache,
+    const int32_t* __restrict__ token_table, int64_t tt_stride, const int32_t* __restrict__ seq_req,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const void* __restrict__ sink, float scale,
+    void* __restrict__ out, int64_t n, int heads, int kv_heads, int dk, int dv) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* sq = lds + wave * (dk + 128);  // [dk] query
+  float* sp = sq + dk;                  // [64] weights of the tile
+  int* sr = (int*)(sp + 64);            // [64] cache rows of the tile
+  const int64_t w = (int64_t)blockIdx.x * 4 + wave;
+  if (w >= n * heads) return;  // (no workgroup barrier below: waves are independent)
+  const int64_t t = w / heads;
+  const int h = (int)(w - t * heads);
+  const int g = h / (heads / kv_heads);
+  const int pos = tok_pos[t];
+  const bool vec = (dk % (DT == LL_F32 ? 4 : 8) == 0) && ((reinterpret_cast<uintptr_t>(k_cache) & 15u) == 0);
+  const int32_t* table = token_table + (int64_t)seq_req[tok_seq[t]] * tt_stride;
+  for (int c = lane; c < dk; c += 64) sq[c] = ldv<DT>(q, (t * heads + h) * dk + c);
+  float m = -INFINITY, l = 0.f;
+  if (sink) {
+    m = ldv<DT>(sink, h);
+    l = 1.0f;
+  }
+  float acc[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) acc[i] = 0.f;
+  __builtin_amdgcn_wave_barrier();
+  for (int base = 0; base <= pos; base += 64) {
+    const int j = base + lane;
+    float s = -INFINITY;
+    int row = 0;
+    if (j <= pos) {
+      row = table[j];
+      const int64_t kb = ((int64_t)row * kv_heads + g) * dk;
+      s = dot_row<DT>(sq, k_cache, kb, dk, vec) * scale;
+    }
+    const float tile_max = wave_max(s);
+    const float m_new = fmaxf(m, tile_max);
+    const float p = j <= pos ? expf(s - m_new) : 0.f;
+    const float corr = m == -INFINITY ? 0.f : expf(m - m_new);
+    l = l * corr + wave_sum(p);
+    m = m_new;
+    sp[lane] = p;
+    sr[lane] = row;
+    __builtin_amdgcn_wave_barrier();
+    const int cnt = pos - base + 1 < 64 ? pos - base + 1 : 64;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int c = lane + 64 * i;
+      float a = acc[i] * corr;
+      if (c < dv) {
+        for (int jj = 0; jj < cnt; ++jj) a += sp[jj] * ldv<DT>(v_cache, ((int64_t)sr[jj] * kv_heads + g) * dv + c);
+      }
+      acc[i] = a;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int c = lane + 64 * i;
+    if (c < dv) stv<DT>(out, (t * heads + h) * dv + c, acc[i] * inv);
+  }
+}
+
+}  // namespace
+
+#define LL_BY_DTYPE(dtype, CALL)             \
+  do {                                       \
+    if (dtype == LL_F16) { CALL(LL_F16); }   \
+    else if (dtype == LL_BF16) { CALL(LL_BF16); } \
+    else { CALL(LL_F32); }                   \
+  } while (0)
+
+extern "C" int ll_qk_norm_cache(const void* qkv, int64_t ld, const void* q_w, const void* k_w, float eps, float temp_coef,
+                                int64_t temp_every, const int32_t* tok_pos, const int32_t* select, void* q_out, void* k_cache,
+                                void* v_cache, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int dtype,
+                                void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || heads < 1 || kv_heads < 1 || heads % kv_heads || dk < 1 || dv < 1 || temp_every < 1 ||
+      ld < (heads + kv_heads) * dk + kv_heads * dv)
+    return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!qkv || !tok_pos || !select || !q_out || !k_cache || !v_cache) return LL_ERR_ARG;
+  const int64_t waves = n * (heads + 2 * kv_heads);
+  const dim3 grid((unsigned)((waves + 3) / 4));
+#define CALL(DT)                                                                                                              \
+  qk_norm_cache_kernel<DT><<<grid, 256, 0, (hipStream_t)stream>>>(qkv, ld, q_w, k_w, eps, temp_coef, (int)temp_every, tok_pos, \
+                                                                 select, q_out, k_cache, v_cache, n, (int)heads, (int)kv_heads, \
+                                                                 (int)dk, (int)dv)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+  return LL_LAUNCH_CHECK();
+}
+
+extern "C" int ll_ragged_attention(const void* q, const void* k_cache, const void* v_cache, const int32_t* token_table,
+                                   int64_t tt_stride, const int32_t* seq_req, const int32_t* tok_seq, const int32_t* tok_pos,
+                                   const void* sink, float scale, void* out, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk,
+                                   int64_t dv, int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || heads < 1 || kv_heads < 1 || heads % kv_heads || dk < 1 || dk > 1024 || dv < 1 || dv > 256) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!q || !k_cache || !v_cache || !token_table || !seq_req || !tok_seq || !tok_pos || !out) return LL_ERR_ARG;
+  const int64_t waves = n * heads;
+  const dim3 grid((unsigned)((waves + 3) / 4));
+  const size_t lds = sizeof(float) * 4 * (size_t)(dk + 128);
+  const int vpl = (int)((dv + 63) / 64);
+  hipStream_t st = (hipStream_t)stream;
+#define CALL_V(DT, V)                                                                                                        \
+  ragged_attention_kernel<DT, V><<<grid, 256, lds, st>>>(q, k_cache, v_cache, token_table, tt_stride, seq_req, tok_seq, tok_pos, \
+                                                         sink, scale, out, n, (int)heads, (int)kv_heads, (int)dk, (int)dv)
+#define CALL(DT)                     \
+  if (vpl == 1) CALL_V(DT, 1);       \
+  else if (vpl == 2) CALL_V(DT, 2);  \
+  else CALL_V(DT, 4)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+#undef CALL_V
+  return LL_LAUNCH_CHECK();
+}

@@ -1,0 +1,363 @@
+// Sequence-mixing layers over RAGGED steps (several sequences, each bringing a run of consecutive tokens: a portion of a
+// prompt, or one decoded token) with a 32-bit residual stream:
+//
+//   ll_add_rmsnorm_shift   residual add (fp32) + RMS norm (fp32) + optional token shift against the previous token's normed
+//                          row (carried per sequence in a state slot) -> activations in the storage dtype
+//   ll_xielu               the xIELU activation with its two learned numbers
+//   ll_cast_pair / ll_residual_set   the two ends of a projection over [x ; x0] that re-enters the residual stream
+//   ll_gated_linear_scan   per-head linear recurrence S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, o_t = S_t^T q_t with a
+//                          lower-bounded forget gate and a per-head RMS norm of o (HGRN2), state in fp32 slots
+//
+// Storage dtype DT = LL_F16 / LL_BF16 / LL_F32 for activations and weights; everything that the recurrence, the norms and
+// the residual touch is fp32.  A step is described by   seq_start[b + 1] (first flat token of each sequence's run),
+// seq_first_pos[b] (position of that token inside its sequence: 0 = the sequence starts here and carries no state yet),
+// seq_slot[b] (state slot), and for per-token kernels tok_seq[n].
+#include "common.h"
+
+namespace {
+
+template <int DT> struct Store { typedef uint16_t type; };
+template <> struct Store<LL_F32> { typedef float type; };
+
+template <int DT>
+__device__ __forceinline__ float ldv(const void* p, int64_t i) {
+  if constexpr (DT == LL_F32) return ((const float*)p)[i];
+  else return to_f32<DT>(((const uint16_t*)p)[i]);
+}
+template <int DT>
+__device__ __forceinline__ void stv(void* p, int64_t i, float v) {
+  if constexpr (DT == LL_F32) ((float*)p)[i] = v;
+  else ((uint16_t*)p)[i] = from_f32<DT>(v);
+}
+
+// sum over a 256-thread workgroup, same order for every caller (wave sums, then the four waves in order): the value a
+// row's norm gets does not depend on which workgroup computes it
+__device__ __forceinline__ float block_sum256(float v, float* lds4) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds4[wave] = v;
+  __syncthreads();
+  return ((lds4[0] + lds4[1]) + lds4[2]) + lds4[3];
+}
+
+// One workgroup per token.  s = x_in + delta (fp32; written to x_out when delta is given), h = s / sqrt(mean(s^2) + eps) * w,
+// y = h + (h_prev - h) * shift, h_prev = the same h of the previous token of the sequence: recomputed from the previous row
+// when that token is part of this step, read from the sequence's state slot when the run starts inside the sequence, zero
+// at position 0.  The last token of a run leaves its h in the other half of the slot pair (state is double-buffered by the
+// per-sequence parity: a run's first token reads while its last token writes).
+template <int DT>
+__global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(
+    const float* __restrict__ x_in, const void* __restrict__ delta, float* __restrict__ x_out, const void* __restrict__ weight,
+    const void* __restrict__ shift, void* __restrict__ y, int64_t n, int width, float eps, const int32_t* __restrict__ tok_seq,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
+    const int32_t* __restrict__ seq_parity, float* __restrict__ state, int64_t state_half) {
+  __shared__ float red[4];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float* xr = x_in + t * width;
+  float ss = 0.f;
+  for (int i = tid; i < width; i += 256) {
+    float s = xr[i];
+    if (delta) s += ldv<DT>(delta, t * width + i);
+    ss += s * s;
+  }
+  ss = block_sum256(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  int mode = 0;  // 0: no shift, 1: previous row of this step, 2: state slot, 3: zeros
+  int b = 0;
+  const float* prev_state = nullptr;
+  float inv_prev = 0.f;
+  if (shift) {
+    b = tok_seq[t];
+    const int start = seq_start[b];
+    if (t > start) {
+      mode = 1;
+      const float* pr = x_in + (t - 1) * width;
+      float sp = 0.f;
+      for (int i = tid; i < width; i += 256) {
+        float s = pr[i];
+        if (delta) s += ldv<DT>(delta, (t - 1) * width + i);
+        sp += s * s;
+      }
+      sp = block_sum256(sp, red);
+      inv_prev = 1.0f / sqrtf(sp / (float)width + eps);
+    } else if (seq_first_pos[b] > 0) {
+      mode = 2;
+      prev_state = state + (int64_t)seq_parity[b] * state_half + (int64_t)seq_slot[b] * width;
+    } else {
+      mode = 3;
+    }
+  }
+  float* keep = nullptr;
+  if (shift && t == seq_start[b + 1] - 1)
+    keep = state + (int64_t)(1 - seq_parity[b]) * state_half + (int64_t)seq_slot[b] * width;
+  for (int i = tid; i < width; i += 256) {
+    float s = xr[i];
+    if (delta) {
+      s += ldv<DT>(delta, t * width + i);
+      x_out[t * width + i] = s;
+    }
+    const float w = ldv<DT>(weight, i);
+    const float h = s * inv * w;
+    float out = h;
+    if (mode) {
+      float hp = 0.f;
+      if (mode == 1) {
+        float s1 = x_in[(t - 1) * width + i];
+        if (delta) s1 += ldv<DT>(delta, (t - 1) * width + i);
+        hp = s1 * inv_prev * w;
+      } else if (mode == 2) {
+        hp = prev_state[i];
+      }
+      out = h + (hp - h) * ldv<DT>(shift, i);
+      if (keep) keep[i] = h;
+    }
+    stv<DT>(y, t * width + i, out);
+  }
+}
+
+__device__ __forceinline__ float softplus_f32(float v) { return v > 20.f ? v : log1pf(expf(v)); }
+
+// xIELU: z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2
+template <int DT>
+__global__ __launch_bounds__(256) void xielu_kernel(void* __restrict__ y, const void* __restrict__ z, const void* __restrict__ pq,
+                                                    int64_t n) {
+  const float ap = softplus_f32(ldv<DT>(pq, 0));
+  const float an = 0.5f + softplus_f32(ldv<DT>(pq, 1));
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const float v = ldv<DT>(z, i);
+    const float r = v > 0.f ? ap * v * v + 0.5f * v : an * (expm1f(v) - v) + 0.5f * v;
+    stv<DT>(y, i, r);
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void cast_pair_kernel(void* __restrict__ out, const float* __restrict__ a,
+                                                        const void* __restrict__ a_delta, const float* __restrict__ b, int64_t n,
+                                                        int width) {
+  const int64_t total = n * 2 * width;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t row = i / (2 * width);
+    const int c = (int)(i - row * 2 * width);
+    float val;
+    if (c < width) {
+      val = a[row * width + c];
+      if (a_delta) val += ldv<DT>(a_delta, row * width + c);
+    } else {
+      val = b[row * width + c - width];
+    }
+    stv<DT>(out, i, val);
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void residual_set_kernel(float* __restrict__ x, const void* __restrict__ y,
+                                                           const void* __restrict__ bias, int64_t n, int width) {
+  const int64_t total = n * width;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    float v = ldv<DT>(y, i);
+    if (bias) v += ldv<DT>(bias, i % width);
+    x[i] = v;
+  }
+}
+
+// --------------------------------------------------------------------------------------------------------------------- //
+// Gated linear recurrence.  One workgroup per (sequence of the step, head).  Thread (g, c): column c of the head's state
+// (c < dv) and rows g, g + KG, ... (KG = 256 / dv column groups), R rows in registers.  Tokens are taken TB at a time:
+// their gates, queries and values are staged in LDS (gate and silu evaluated once, in fp32), every thread walks the TB
+// tokens over its rows (state update + partial o), the partials of the KG groups are added in group order, o is RMS-normed
+// over dv and stored.  The state is read when the run starts inside the sequence (first_pos > 0), zero otherwise, and
+// written back at the end of the run.
+// --------------------------------------------------------------------------------------------------------------------- //
+constexpr int kScanTB = 8;
+
+template <int DT, int RMAX>
+__global__ __launch_bounds__(256) void gated_linear_scan_kernel(
+    const void* __restrict__ q, const void* __restrict__ f, const void* __restrict__ v, int64_t ld, const void* __restrict__ f_bias,
+    const void* __restrict__ lower, const void* __restrict__ norm_w, float eps, void* __restrict__ out, int heads, int dk, int dv,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
+    float* __restrict__ state) {
+  extern __shared__ float lds[];
+  const int b = blockIdx.x, head = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int kg = 256 / dv > 0 ? (256 / dv < dk ? 256 / dv : dk) : 1;
+  const int c = tid % dv, g = tid / dv;
+  const bool active = g < kg;
+  const int rows = active ? (dk - g + kg - 1) / kg : 0;  // rows g, g + kg, ...
+  float* sf = lds;                        // [TB][dk] forget gates
+  float* sq = sf + kScanTB * dk;          // [TB][dk] queries
+  float* sv = sq + kScanTB * dk;          // [TB][dv] values
+  float* sp = sv + kScanTB * dv;          // [TB][kg][dv] partial outputs
+  float* so = sp + kScanTB * kg * dv;     // [TB][dv] outputs
+  float* sn = so + kScanTB * dv;          // [TB] inverse rms
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  float* st = state + ((int64_t)seq_slot[b] * heads + head) * dk * dv;
+  float S[RMAX];
+  const bool carry = seq_first_pos[b] > 0;
+#pragma unroll
+  for (int r = 0; r < RMAX; ++r) S[r] = (r < rows && carry) ? st[(int64_t)(g + r * kg) * dv + c] : 0.f;
+  for (int base = t0; base < t1; base += kScanTB) {
+    const int nt = t1 - base < kScanTB ? t1 - base : kScanTB;
+    __syncthreads();
+    for (int i = tid; i < nt * dk; i += 256) {
+      const int tt = i / dk, k = i - tt * dk;
+      const int64_t at = (int64_t)(base + tt) * ld + head * dk + k;
+      const float lo = ldv<DT>(lower, head * dk + k);
+      const float raw = ldv<DT>(f, at) + ldv<DT>(f_bias, head * dk + k);
+      const float sig = 1.0f / (1.0f + expf(-raw));
+      sf[i] = lo + (1.0f - lo) * sig;
+      const float qv = ldv<DT>(q, at);
+      sq[i] = qv / (1.0f + expf(-qv));
+    }
+    for (int i = tid; i < nt * dv; i += 256) {
+      const int tt = i / dv, cc = i - tt * dv;
+      sv[i] = ldv<DT>(v, (int64_t)(base + tt) * ld + head * dv + cc);
+    }
+    __syncthreads();
+    if (active) {
+      for (int tt = 0; tt < nt; ++tt) {
+        const float val = sv[tt * dv + c];
+        float acc = 0.f;
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) {
+          if (r < rows) {
+            const int k = g + r * kg;
+            const float fg = sf[tt * dk + k];
+            S[r] = fg * S[r] + (1.0f - fg) * val;
+            acc += S[r] * sq[tt * dk + k];
+          }
+        }
+        sp[(tt * kg + g) * dv + c] = acc;
+      }
+    }
+    __syncthreads();
+    for (int i = tid; i < nt * dv; i += 256) {
+      const int tt = i / dv, cc = i - tt * dv;
+      float o = 0.f;
+      for (int gg = 0; gg < kg; ++gg) o += sp[(tt * kg + gg) * dv + cc];
+      so[i] = o;
+    }
+    __syncthreads();
+    {
+      // one wave per token: mean of squares over dv in lane order
+      const int wave = tid >> 6, lane = tid & 63;
+      for (int tt = wave; tt < nt; tt += 4) {
+        float ss = 0.f;
+        for (int cc = lane; cc < dv; cc += 64) ss += so[tt * dv + cc] * so[tt * dv + cc];
+        ss = wave_sum(ss);
+        if (lane == 0) sn[tt] = 1.0f / sqrtf(ss / (float)dv + eps);
+      }
+    }
+    __syncthreads();
+    for (int i = tid; i < nt * dv; i += 256) {
+      const int tt = i / dv, cc = i - tt * dv;
+      stv<DT>(out, ((int64_t)(base + tt) * heads + head) * dv + cc, so[i] * sn[tt] * ldv<DT>(norm_w, cc));
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RMAX; ++r)
+    if (r < rows) st[(int64_t)(g + r * kg) * dv + c] = S[r];
+}
+
+inline unsigned flat_grid(int64_t total) {
+  const int64_t g = (total + 255) / 256;
+  return (unsigned)(g < 1 ? 1 : (g > 16384 ? 16384 : g));
+}
+
+}  // namespace
+
+#define LL_BY_DTYPE(dtype, CALL)             \
+  do {                                       \
+    if (dtype == LL_F16) { CALL(LL_F16); }   \
+    else if (dtype == LL_BF16) { CALL(LL_BF16); } \
+    else { CALL(LL_F32); }                   \
+  } while (0)
+
+extern "C" int ll_add_rmsnorm_shift(const float* x_in, const void* delta, float* x_out, const void* weight, const void* shift,
+                                    void* y, int64_t n, int64_t width, float eps, const int32_t* tok_seq,
+                                    const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot,
+                                    const int32_t* seq_parity, float* state, int64_t state_half, int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || width < 1 || width > (1 << 20)) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!x_in || !weight || !y || (delta && !x_out)) return LL_ERR_ARG;
+  if (delta && x_out == x_in && shift) return LL_ERR_ARG;  // the previous row is re-read: it must still hold the old sum
+  if (shift && (!tok_seq || !seq_start || !seq_first_pos || !seq_slot || !seq_parity || !state)) return LL_ERR_ARG;
+#define CALL(DT)                                                                                                          \
+  add_rmsnorm_shift_kernel<DT><<<dim3((unsigned)n), 256, 0, (hipStream_t)stream>>>(                                         \
+      x_in, delta, x_out, weight, shift, y, n, (int)width, eps, tok_seq, seq_start, seq_first_pos, seq_slot, seq_parity, state, \
+      state_half)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+  return LL_LAUNCH_CHECK();
+}
+
+extern "C" int ll_xielu(void* y, const void* z, const void* pq, int64_t n, int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!y || !z || !pq) return LL_ERR_ARG;
+#define CALL(DT) xielu_kernel<DT><<<dim3(flat_grid(n)), 256, 0, (hipStream_t)stream>>>(y, z, pq, n)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+  return LL_LAUNCH_CHECK();
+}
+
+extern "C" int ll_cast_pair(void* out, const float* a, const void* a_delta, const float* b, int64_t n, int64_t width, int dtype,
+                            void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || width < 1 || width > (1 << 20)) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!out || !a || !b) return LL_ERR_ARG;
+#define CALL(DT) cast_pair_kernel<DT><<<dim3(flat_grid(n * 2 * width)), 256, 0, (hipStream_t)stream>>>(out, a, a_delta, b, n, (int)width)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+  return LL_LAUNCH_CHECK();
+}
+
+extern "C" int ll_residual_set(float* x, const void* y, const void* bias, int64_t n, int64_t width, int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || width < 1 || width > (1 << 20)) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!x || !y) return LL_ERR_ARG;
+#define CALL(DT) residual_set_kernel<DT><<<dim3(flat_grid(n * width)), 256, 0, (hipStream_t)stream>>>(x, y, bias, n, (int)width)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+  return LL_LAUNCH_CHECK();
+}
+
+extern "C" int ll_gated_linear_scan_supported(int64_t dk, int64_t dv) {
+  if (dk < 1 || dv < 1 || dv > 256) return 0;
+  const int64_t kg = 256 / dv < dk ? 256 / dv : dk;
+  return (dk + kg - 1) / kg <= 64 ? 1 : 0;
+}
+
+extern "C" int ll_gated_linear_scan(const void* q, const void* f, const void* v, int64_t ld, const void* f_bias, const void* lower,
+                                    const void* norm_w, float eps, void* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
+                                    const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, float* state,
+                                    int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (batch < 0 || heads < 1 || heads > 65535 || !ll_gated_linear_scan_supported(dk, dv)) return LL_ERR_SHAPE;
+  if (batch == 0) return LL_OK;
+  if (!q || !f || !v || !f_bias || !lower || !norm_w || !out || !seq_start || !seq_first_pos || !seq_slot || !state)
+    return LL_ERR_ARG;
+  const int kg = (int)(256 / dv < dk ? 256 / dv : dk);
+  const int rmax = (int)((dk + kg - 1) / kg);
+  const size_t lds = sizeof(float) * (size_t)(kScanTB * (2 * dk + dv) + kScanTB * kg * dv + kScanTB * dv + kScanTB);
+  if (lds > 64 * 1024) return LL_ERR_SHAPE;
+  const dim3 grid((unsigned)batch, (unsigned)heads);
+  hipStream_t st = (hipStream_t)stream;
+#define CALL_R(DT, R)                                                                                                        \
+  gated_linear_scan_kernel<DT, R><<<grid, 256, lds, st>>>(q, f, v, ld, f_bias, lower, norm_w, eps, out, (int)heads, (int)dk, \
+                                                          (int)dv, seq_start, seq_first_pos, seq_slot, state)
+#define CALL(DT)                       \
+  if (rmax <= 4) CALL_R(DT, 4);        \
+  else if (rmax <= 16) CALL_R(DT, 16); \
+  else if (rmax <= 32) CALL_R(DT, 32); \
+  else CALL_R(DT, 64)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+#undef CALL_R
+  return LL_LAUNCH_CHECK();
+}

@@ -21,14 +21,17 @@ class PagedKVPool:
         self.block_size, self.num_blocks, self.device = block_size, num_blocks, device
         self.max_requests, self.max_seq_len = max_requests, max_seq_len
         self.max_tokens = num_blocks * block_size
-        self.kv_buffer = [torch.zeros(self.max_tokens, 2 * num_kv_heads, head_dim, dtype=dtype, device=device)
-                          for _ in range(num_layers)]
+        self.kv_buffer = self._make_buffers(num_layers, num_kv_heads, head_dim, dtype)
         self.blocks_per_request = (max_seq_len + block_size - 1) // block_size
         self.free_stack = torch.empty(num_blocks - 1, dtype=torch.int32, device=device)
         self.state = torch.zeros(2, dtype=torch.int32, device=device)          # [free blocks, error flags]
         self.block_table = torch.zeros(max_requests, self.blocks_per_request, dtype=torch.int32, device=device)
         self.req_blocks = torch.zeros(max_requests, dtype=torch.int32, device=device)
         self.reset()
+
+    def _make_buffers(self, num_layers, num_kv_heads, head_dim, dtype):
+        return [torch.zeros(self.max_tokens, 2 * num_kv_heads, head_dim, dtype=dtype, device=self.device)
+                for _ in range(num_layers)]
 
     def reset(self) -> None:
         L.check(L.lib().ll_kv_paged_reset(self.free_stack.data_ptr(), self.state.data_ptr(), self.req_blocks.data_ptr(),
@@ -88,3 +91,52 @@ class PagedKVPool:
         self.state.copy_(snap[0])
         self.req_blocks.copy_(snap[1])
         self.block_table.copy_(snap[2])
+
+
+class PagedStateCache(PagedKVPool):
+    """Cache of a model whose layer RUNS differ in what they keep per sequence (a layer that runs several times in a forward
+    pass keeps one set per run): attention runs own ``(K [rows, kv_heads, dk], V [rows, kv_heads, dv])`` in the block pool --
+    key and value widths may differ --, recurrent runs own a fixed-size fp32 state ``[slots, heads, dk, dv]``, and any run may
+    own a token-shift row pair ``[2, slots, width]`` (double-buffered by the sequence's parity).  One block allocator, one
+    block table and one per-token row table serve all attention runs; a sequence's slot is its row of those tables, so blocks
+    and slots are handed out and given back together.  Fixed-size state is never cleared: the kernels start a sequence whose
+    run begins at position 0 from zeros, whatever an earlier owner of the slot left."""
+
+    def __init__(self, runs, num_blocks: int, block_size: int, device, max_requests: int, max_seq_len: int, dtype):
+        """``runs``: one mapping per layer run: ``{"kind": "attention", "kv_heads", "dk", "dv"}`` or
+        ``{"kind": "recurrent", "heads", "dk", "dv"}``, each with an optional ``"shift_width"``."""
+        self.runs = [dict(r) for r in runs]
+        self.dtype = dtype
+        super().__init__(len(self.runs), num_blocks, block_size, 1, 1, device, max_requests, max_seq_len, dtype)
+
+    def _make_buffers(self, num_layers, num_kv_heads, head_dim, dtype):
+        dev, slots = self.device, self.max_requests
+        self.recurrent, self.shift = [], []
+        buffers = []
+        for r in self.runs:
+            if r["kind"] == "attention":
+                buffers.append((torch.zeros(self.max_tokens, r["kv_heads"], r["dk"], dtype=dtype, device=dev),
+                                torch.zeros(self.max_tokens, r["kv_heads"], r["dv"], dtype=dtype, device=dev)))
+                self.recurrent.append(None)
+            elif r["kind"] == "recurrent":
+                buffers.append(None)
+                self.recurrent.append(torch.zeros(slots, r["heads"], r["dk"], r["dv"], dtype=torch.float32, device=dev))
+            else:
+                raise ValueError(f"unknown layer-run kind {r['kind']!r}")
+            w = int(r.get("shift_width", 0))
+            self.shift.append(torch.zeros(2, slots, w, dtype=torch.float32, device=dev) if w else None)
+        return buffers
+
+    def extend(self, req_idx: torch.Tensor, new_lens: torch.Tensor, longest_run: int, token_table: torch.Tensor) -> torch.Tensor:
+        """Blocks for every listed request up to ``new_lens[i]`` tokens; returns the cache rows of each request's LAST
+        ``longest_run`` positions ``[n, longest_run]`` (a request that brings fewer tokens uses the tail of its row)."""
+        return self._extend(req_idx, new_lens, 0, longest_run, 1, token_table).view(req_idx.numel(), longest_run)
+
+    def state_bytes(self) -> int:
+        total = 0
+        for group in (self.kv_buffer, self.recurrent, self.shift):
+            for t in group:
+                for u in (t if isinstance(t, tuple) else (t,)):
+                    if u is not None:
+                        total += u.numel() * u.element_size()
+        return total

@@ -1,0 +1,159 @@
+"""Ragged steps: the step function of models that take SEVERAL sequences per forward pass, each bringing a run of consecutive
+tokens -- a portion of a prompt of any length, or the one token it decoded last -- against the cache and state that earlier
+steps left.  Where :class:`SlotBatch` (slots.py) drives the padded-grid prefill / lockstep decode of the llama-shaped models,
+this drives the layered models (model_layers.py): one flat token array, no padding, prompt portions next to decode tokens.
+
+:class:`RaggedStep` is the metadata every kernel of such a step reads; :class:`RaggedRunner` owns the model, its
+:class:`PagedStateCache` and the request slots, and is what both the generation engine (engine.py) and the trace replay
+(trace_replay.py) call.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Sequence
+from dataclasses import dataclass
+
+import torch
+
+from .paged_kv import PagedStateCache
+
+
+@dataclass
+class RaggedStep:
+    """Device-side description of one step (all int32).  Per token: ``tok_seq`` (index of its sequence in the step), ``tok_pos``
+    (position inside its sequence), ``select`` (cache row it writes).  Per sequence: ``seq_start [b + 1]`` (its run in the flat
+    arrays), ``seq_first_pos`` (position of the run's first token), ``seq_slot`` / ``seq_req`` (its state slot = its row of the
+    block and token tables), ``seq_parity`` (which half of a double-buffered state pair it reads)."""
+
+    num_tokens: int
+    num_seqs: int
+    tok_seq: torch.Tensor
+    tok_pos: torch.Tensor
+    select: torch.Tensor
+    seq_start: torch.Tensor
+    seq_first_pos: torch.Tensor
+    seq_slot: torch.Tensor
+    seq_parity: torch.Tensor
+
+    @property
+    def seq_req(self) -> torch.Tensor:
+        return self.seq_slot
+
+
+class RaggedRunner:
+    """Model + cache + request slots.  ``admit()`` hands out a slot, ``step()`` runs one ragged step and returns the logits of
+    the asked rows, ``release()`` gives a request's blocks and slot back.  Nothing is kept per request on the host but its
+    length and parity; blocks are popped and pushed on the device (``PagedStateCache``)."""
+
+    def __init__(self, model, max_tokens: int, max_requests: int = 4, block_size: int = 64, device="cuda",
+                 max_seq_len: int | None = None):
+        """``max_tokens``: the most tokens that live requests hold at any time, each request's count rounded up to a multiple
+        of ``block_size``: the block pool is made for that many (plus the junk block), not for ``max_requests`` full-length
+        sequences."""
+        self.model = model
+        self.device = torch.device(device)
+        self.block_size = block_size
+        blocks = -(-max_tokens // block_size)
+        self.max_seq_len = (max_seq_len if max_seq_len is not None else blocks * block_size)
+        self.max_seq_len = -(-self.max_seq_len // block_size) * block_size
+        self.max_requests = max_requests
+        self.cache = PagedStateCache(model.cache_runs(), blocks + 1, block_size, self.device, max_requests, self.max_seq_len,
+                                     model.dtype)
+        self.token_table = torch.zeros(max_requests, self.max_seq_len, dtype=torch.int32, device=self.device)
+        self.total_blocks = blocks
+        self._free_slots = list(range(max_requests))
+        self._len: dict[int, int] = {}
+        self._parity: dict[int, int] = {}
+
+    # ------------------------------------------------------------------ requests ---- #
+    @property
+    def free_slots(self) -> int:
+        return len(self._free_slots)
+
+    def blocks_held(self) -> int:
+        return sum(-(-n // self.block_size) for n in self._len.values())
+
+    def blocks_for(self, tokens: int) -> int:
+        return -(-tokens // self.block_size)
+
+    def length(self, slot: int) -> int:
+        return self._len[slot]
+
+    def admit(self) -> int:
+        if not self._free_slots:
+            raise RuntimeError(f"all {self.max_requests} request slots are taken")
+        slot = self._free_slots.pop(0)
+        self._len[slot] = 0
+        self._parity[slot] = 0
+        return slot
+
+    def release(self, slots: Sequence[int]) -> None:
+        slots = [s for s in slots if s in self._len]
+        if not slots:
+            return
+        self.cache.release(torch.tensor(slots, dtype=torch.int32, device=self.device))
+        for s in slots:
+            del self._len[s], self._parity[s]
+            self._free_slots.append(s)
+
+    # ------------------------------------------------------------------ one step ---- #
+    def build_step(self, entries: Sequence[tuple[int, Sequence[int]]]) -> tuple[RaggedStep, torch.Tensor]:
+        """``entries``: ``(slot, next tokens)`` per sequence, every slot at most once.  Reserves blocks for the new tokens and
+        advances the host-side lengths and parities."""
+        if not entries:
+            raise ValueError("an empty step")
+        slots = [s for s, _ in entries]
+        if len(set(slots)) != len(slots):
+            raise ValueError("a request rides at most once in a step")
+        counts = [len(t) for _, t in entries]
+        if min(counts) < 1:
+            raise ValueError("every entry brings at least one token")
+        first = [self._len[s] for s in slots]
+        new_len = [f + c for f, c in zip(first, counts)]
+        if max(new_len) > self.max_seq_len:
+            raise RuntimeError(f"a sequence of {max(new_len)} tokens exceeds the cache's {self.max_seq_len}")
+        need = sum(self.blocks_for(n) - self.blocks_for(f) for n, f in zip(new_len, first))
+        if self.blocks_held() + need > self.total_blocks:
+            raise RuntimeError(f"the block pool is exhausted: {self.blocks_held()} of {self.total_blocks} blocks held, {need} more asked")
+        starts, tok_seq, tok_pos, pick, tokens = [0], [], [], [], []
+        longest = max(counts)
+        for i, ((_, toks), f, c) in enumerate(zip(entries, first, counts)):
+            starts.append(starts[-1] + c)
+            tok_seq += [i] * c
+            tok_pos += range(f, f + c)
+            pick += range(i * longest + longest - c, (i + 1) * longest)
+            tokens += [int(t) for t in toks]
+        dev = self.device
+
+        def vec(values):
+            return torch.tensor(values, dtype=torch.int32, device=dev)
+
+        seq_slot = vec(slots)
+        rows = self.cache.extend(seq_slot, vec(new_len), longest, self.token_table)
+        select = rows.reshape(-1)[torch.tensor(pick, dtype=torch.long, device=dev)].contiguous()
+        step = RaggedStep(num_tokens=len(tokens), num_seqs=len(entries), tok_seq=vec(tok_seq), tok_pos=vec(tok_pos), select=select,
+                          seq_start=vec(starts), seq_first_pos=vec(first), seq_slot=seq_slot,
+                          seq_parity=vec([self._parity[s] for s in slots]))
+        for s, n in zip(slots, new_len):
+            self._len[s] = n
+            self._parity[s] ^= 1
+        return step, torch.tensor(tokens, dtype=torch.long, device=dev)
+
+    @torch.no_grad()
+    def step(self, entries: Sequence[tuple[int, Sequence[int]]], logits_rows: Sequence[int] | None = None, *,
+             collect_layers: list | None = None) -> torch.Tensor | None:
+        """Run the entries as ONE batch.  ``logits_rows``: flat token indices (in entry order) whose logits are wanted; ``None``
+        = the last token of every entry; an empty list = none (the step still fills cache and state).  Returns
+        ``[rows, vocab]`` logits in the model's dtype, or ``None``."""
+        step, token_ids = self.build_step(entries)
+        if logits_rows is None:
+            logits_rows = [int(v) - 1 for v in step.seq_start.tolist()[1:]]
+        rows = torch.tensor(list(logits_rows), dtype=torch.long, device=self.device) if len(logits_rows) else None
+        out = self.model(token_ids, step, self.cache, self.token_table, logits_rows=rows, collect_layers=collect_layers)
+        return out
+
+    def check_errors(self) -> None:
+        """Synchronising read of the block pool's sticky error word."""
+        err = self.cache.error
+        if err:
+            raise RuntimeError(f"paged cache reported error bits {err:#x} (1: too few free blocks, 2: a request outgrew its table row)")

@@ -38,3 +38,17 @@ def tanh(x):
 @torch.no_grad()
 def gelu(x):
     return _apply(x, 3, "gelu")
+
+
+@torch.no_grad()
+def xielu(z: torch.Tensor, pq: torch.Tensor) -> torch.Tensor:
+    """xIELU with its two learned numbers ``pq = (p, q)``: ``softplus(p) z^2 + z / 2`` for ``z > 0``, else
+    ``(1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2``; fp32 arithmetic, one rounding to the storage dtype (fp16 / bf16 / fp32)."""
+    L.require_cuda(z, pq)
+    if pq.dtype != z.dtype or pq.numel() != 2:
+        raise ValueError("xielu: pq holds the two numbers (p, q) in the activations' dtype")
+    zc = z.contiguous()
+    y = torch.empty_like(zc)
+    L.check(L.lib().ll_xielu(y.data_ptr(), zc.data_ptr(), pq.contiguous().data_ptr(), zc.numel(), L.dtype_code(z.dtype),
+                             L.stream_ptr()), "xielu")
+    return y.view(z.shape)

@@ -277,3 +277,57 @@ def flash_attention2_no_pad(q, k, v, sm_scale, b_start_loc, b_seq_len, max_seq_l
         "flash_attention2_no_pad",
     )
     return output
+
+
+# ------------------------------------------------------------------------------------- #
+# ragged steps against a paged cache with separate key / value widths (csrc/ragged_attn.hip)
+# ------------------------------------------------------------------------------------- #
+@torch.no_grad()
+def qk_norm_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, q_weight, k_weight, eps: float, temp_coef: float,
+                  temp_every: int, step, k_cache, v_cache):
+    """Fused projection rows ``[q | k | v]`` -> queries ``[n, heads, dk]`` (per-head RMS norm, then the position temperature
+    ``1 + temp_coef ln(floor((pos + 1) / temp_every) + 1)``); normed keys and values land in the cache rows ``step.select``."""
+    L.require_cuda(qkv, k_cache, v_cache)
+    n, dt = qkv.shape[0], qkv.dtype
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < (heads + kv_heads) * dk + kv_heads * dv:
+        raise ValueError("qk_norm_cache: rows hold [q | k | v]")
+    if k_cache.dtype != dt or v_cache.dtype != dt or tuple(k_cache.shape[1:]) != (kv_heads, dk) \
+            or tuple(v_cache.shape[1:]) != (kv_heads, dv) or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("qk_norm_cache: caches are contiguous [rows, kv_heads, dk] / [rows, kv_heads, dv] in the rows' dtype")
+    for w in (q_weight, k_weight):
+        if w is not None and (w.dtype != dt or w.numel() != dk or not w.is_contiguous()):
+            raise ValueError("qk_norm_cache: norm weights are [dk] in the rows' dtype")
+    if step.num_tokens != n:
+        raise ValueError("qk_norm_cache: the step describes another number of tokens")
+    q = torch.empty(n, heads, dk, dtype=dt, device=qkv.device)
+    L.check(L.lib().ll_qk_norm_cache(qkv.data_ptr(), qkv.stride(0), L.ptr(q_weight), L.ptr(k_weight), float(eps), float(temp_coef),
+                                     int(temp_every), step.tok_pos.data_ptr(), step.select.data_ptr(), q.data_ptr(),
+                                     k_cache.data_ptr(), v_cache.data_ptr(), n, heads, kv_heads, dk, dv, L.dtype_code(dt),
+                                     L.stream_ptr()), "qk_norm_cache")
+    return q
+
+
+@torch.no_grad()
+def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=None):
+    """Causal softmax attention of every token of a ragged step against positions ``0 .. its own`` of its sequence, keys and
+    values read through ``token_table[request][position]``; ``sink [heads]`` adds ``exp(sink_h)`` to each head's denominator.
+    Scores, weights and the output sum are fp32.  Returns ``[n, heads * dv]``."""
+    L.require_cuda(q, k_cache, v_cache, token_table)
+    n, heads, dk = q.shape
+    kv_heads, dv = v_cache.shape[1], v_cache.shape[2]
+    dt = q.dtype
+    if not q.is_contiguous() or k_cache.dtype != dt or v_cache.dtype != dt or k_cache.shape[1:] != (kv_heads, dk) \
+            or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("ragged_attention: q [n, heads, dk], caches [rows, kv_heads, dk] / [rows, kv_heads, dv], one dtype")
+    if token_table.dtype != torch.int32 or token_table.stride(1) != 1:
+        raise ValueError("ragged_attention: the token table is row-major int32")
+    if sink is not None and (sink.dtype != dt or sink.numel() != heads or not sink.is_contiguous()):
+        raise ValueError("ragged_attention: sink is [heads] in the queries' dtype")
+    if step.num_tokens != n:
+        raise ValueError("ragged_attention: the step describes another number of tokens")
+    out = torch.empty(n, heads * dv, dtype=dt, device=q.device)
+    L.check(L.lib().ll_ragged_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), token_table.data_ptr(),
+                                        token_table.stride(0), step.seq_req.data_ptr(), step.tok_seq.data_ptr(),
+                                        step.tok_pos.data_ptr(), L.ptr(sink), float(scale), out.data_ptr(), n, heads, kv_heads, dk,
+                                        dv, L.dtype_code(dt), L.stream_ptr()), "ragged_attention")
+    return out

@@ -345,3 +345,71 @@ def rope_and_cache(q, kv, cos, sin, batch_size, seq_len, select_index, kv_buffer
         "rope_and_cache",
     )
     return q, kv
+
+
+# ------------------------------------------------------------------------------------- #
+# 32-bit residual stream over ragged steps (csrc/seq_mix.hip)
+# ------------------------------------------------------------------------------------- #
+@torch.no_grad()
+def add_rmsnorm_shift(x_in, delta, weight, eps, *, x_out=None, shift=None, step=None, state=None):
+    """``s = x_in + delta`` (fp32 residual ``[n, width]``; ``delta`` in the storage dtype or ``None``), RMS norm with ``weight``,
+    and -- with ``shift`` -- the token shift ``h + (h_prev - h) * shift`` against the previous token's normed row of the same
+    sequence (``step``: the ragged step's vectors; ``state``: fp32 ``[2, slots, width]`` of this layer run, the half named by the
+    sequence's parity is read, the other written).  Returns ``(y, residual)``: ``y`` in the storage dtype, ``residual`` the
+    tensor that now holds ``s`` (``x_out``, or ``x_in`` when there is no ``delta``)."""
+    L.require_cuda(x_in, weight)
+    n, width = x_in.shape
+    if x_in.dtype != torch.float32 or not x_in.is_contiguous():
+        raise ValueError("add_rmsnorm_shift: the residual stream is contiguous fp32")
+    dt = weight.dtype
+    if delta is not None:
+        if delta.dtype != dt or delta.shape != x_in.shape or not delta.is_contiguous():
+            raise ValueError("add_rmsnorm_shift: delta must match the residual's shape, in the weights' dtype")
+        if x_out is None:
+            x_out = torch.empty_like(x_in)
+        if x_out.data_ptr() == x_in.data_ptr() and shift is not None:
+            raise ValueError("add_rmsnorm_shift: with a token shift the sum goes to another buffer (the previous row is re-read)")
+    y = torch.empty(n, width, dtype=dt, device=x_in.device)
+    if shift is not None:
+        if step is None or state is None or state.dtype != torch.float32 or state.dim() != 3 or state.shape[0] != 2 \
+                or state.shape[2] != width or not state.is_contiguous() or shift.dtype != dt:
+            raise ValueError("add_rmsnorm_shift: the token shift needs the step's vectors and an fp32 [2, slots, width] state")
+        if step.num_tokens != n:
+            raise ValueError("add_rmsnorm_shift: the step describes another number of tokens")
+    L.check(L.lib().ll_add_rmsnorm_shift(
+        x_in.data_ptr(), L.ptr(delta), L.ptr(x_out) if delta is not None else 0, weight.data_ptr(), L.ptr(shift), y.data_ptr(),
+        n, width, float(eps), *( (step.tok_seq.data_ptr(), step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(),
+                                  step.seq_slot.data_ptr(), step.seq_parity.data_ptr(), state.data_ptr(), state.shape[1] * width)
+                                 if shift is not None else (0, 0, 0, 0, 0, 0, 0) ),
+        L.dtype_code(dt), L.stream_ptr()), "add_rmsnorm_shift")
+    return y, (x_out if delta is not None else x_in)
+
+
+@torch.no_grad()
+def cast_pair(a: torch.Tensor, b: torch.Tensor, dtype, a_delta: torch.Tensor | None = None) -> torch.Tensor:
+    """``[a + a_delta | b]`` of two fp32 ``[n, width]`` tensors (``a_delta``: a pending residual update in ``dtype``), cast to
+    ``dtype``: the input of a projection over the pair."""
+    L.require_cuda(a, b)
+    if a_delta is not None and (a_delta.dtype != dtype or a_delta.shape != a.shape or not a_delta.is_contiguous()):
+        raise ValueError("cast_pair: the pending update matches a's shape, in the output dtype")
+    if a.dtype != torch.float32 or b.dtype != torch.float32 or a.shape != b.shape or not (a.is_contiguous() and b.is_contiguous()):
+        raise ValueError("cast_pair: two contiguous fp32 tensors of one shape")
+    n, width = a.shape
+    out = torch.empty(n, 2 * width, dtype=dtype, device=a.device)
+    L.check(L.lib().ll_cast_pair(out.data_ptr(), a.data_ptr(), L.ptr(a_delta), b.data_ptr(), n, width, L.dtype_code(dtype), L.stream_ptr()),
+            "cast_pair")
+    return out
+
+
+@torch.no_grad()
+def residual_set(y: torch.Tensor, bias: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """A projection's rows ``y`` (+ ``bias [width]``) become the fp32 residual stream."""
+    L.require_cuda(y)
+    n, width = y.shape
+    if not y.is_contiguous() or (bias is not None and (bias.dtype != y.dtype or bias.numel() != width or not bias.is_contiguous())):
+        raise ValueError("residual_set: contiguous rows and a bias of their width and dtype")
+    if out is None:
+        out = torch.empty(n, width, dtype=torch.float32, device=y.device)
+    L.check(L.lib().ll_residual_set(out.data_ptr(), y.data_ptr(), L.ptr(bias), n, width, L.dtype_code(y.dtype), L.stream_ptr()),
+            "residual_set")
+    return out

@@ -550,7 +550,7 @@ def dense16_rows_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tenso
     on the row-group weight-streaming kernel (csrc/gemm_w16_rows.hip): finished outputs in one launch, no planes.  ``None`` when
     the call is not served (shape / dtype / alignment, ``LL_DENSE16_ROWS_OFF``): the caller keeps its route."""
     if (not x.is_cuda or x.dtype not in (torch.float16, torch.bfloat16) or weight.dtype != x.dtype or weight.dim() != 2
-            or os.environ.get("LL_DENSE16_ROWS_OFF")):
+            or os.environ.get("LL_DENSE16_ROWS_OFF") or not L.has("ll_dense16_rows_matmul")):
         return None
     n, k = weight.shape
     if x.shape[-1] != k or (bias is not None and (bias.dtype != x.dtype or bias.numel() != n or gate_up_swiglu)):
@@ -577,7 +577,7 @@ def dense16_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | N
     if policy == "auto" and x.shape[-1] and not dense16_wins(x.numel() // x.shape[-1], weight.shape[0], weight.shape[1]):
         return None
     if (not x.is_cuda or x.dtype not in (torch.float16, torch.bfloat16) or weight.dtype != x.dtype or weight.dim() != 2
-            or os.environ.get("LL_DENSE16_OFF")):
+            or os.environ.get("LL_DENSE16_OFF") or not L.has("ll_dense16_matmul")):
         return None
     n, k = weight.shape
     if x.shape[-1] != k or (bias is not None and (bias.dtype != x.dtype or bias.numel() != n)):

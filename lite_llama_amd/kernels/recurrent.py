@@ -1,0 +1,45 @@
+"""Recurrent sequence mixers over ragged steps (csrc/seq_mix.hip): fixed-size fp32 state per (sequence slot, head), carried
+from step to step -- the counterpart, for layers without a growing cache, of the attention kernels next door."""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _lib as L
+
+
+def gated_linear_scan_supported(dk: int, dv: int) -> bool:
+    return bool(L.lib().ll_gated_linear_scan_supported(dk, dv))
+
+
+@torch.no_grad()
+def gated_linear_scan(qfv: torch.Tensor, heads: int, dk: int, dv: int, f_bias, lower, norm_weight, eps: float, step,
+                      state: torch.Tensor) -> torch.Tensor:
+    """HGRN2-style gated linear attention.  ``qfv [n, 2 heads dk + heads dv]`` = the fused projection rows
+    ``[q_raw | f_raw | v]``; per head ``f = lower + (1 - lower) sigmoid(f_raw + f_bias)``,
+    ``S <- diag(f) S + (1 - f) v^T``, ``o = S^T silu(q_raw)``, then ``o`` RMS-normed over ``dv`` with ``norm_weight``.
+    ``state [slots, heads, dk, dv]`` fp32: a sequence whose run starts at position 0 starts from zeros (whatever an earlier
+    owner of the slot left), every run leaves its final state.  Returns ``[n, heads dv]`` in the storage dtype."""
+    L.require_cuda(qfv, f_bias, lower, norm_weight, state)
+    n = qfv.shape[0]
+    dt = qfv.dtype
+    if qfv.dim() != 2 or qfv.stride(1) != 1 or qfv.shape[1] < 2 * heads * dk + heads * dv:
+        raise ValueError("gated_linear_scan: qfv rows hold [q | f | v]")
+    if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (heads, dk, dv):
+        raise ValueError("gated_linear_scan: state is contiguous fp32 [slots, heads, dk, dv]")
+    for t, size in ((f_bias, heads * dk), (lower, heads * dk), (norm_weight, dv)):
+        if t.dtype != dt or t.numel() != size or not t.is_contiguous():
+            raise ValueError("gated_linear_scan: gate bias / lower bound [heads dk] and norm weight [dv] in the rows' dtype")
+    if step.num_tokens != n:
+        raise ValueError("gated_linear_scan: the step describes another number of tokens")
+    if not gated_linear_scan_supported(dk, dv):
+        raise ValueError(f"gated_linear_scan: head geometry {dk} x {dv} is not served (dv <= 256, <= 64 state rows per thread)")
+    out = torch.empty(n, heads * dv, dtype=dt, device=qfv.device)
+    es = qfv.element_size()
+    base = qfv.data_ptr()
+    L.check(L.lib().ll_gated_linear_scan(
+        base, base + heads * dk * es, base + 2 * heads * dk * es, qfv.stride(0), f_bias.data_ptr(), lower.data_ptr(),
+        norm_weight.data_ptr(), float(eps), out.data_ptr(), step.num_seqs, heads, dk, dv, step.seq_start.data_ptr(),
+        step.seq_first_pos.data_ptr(), step.seq_slot.data_ptr(), state.data_ptr(), L.dtype_code(dt), L.stream_ptr()),
+        "gated_linear_scan")
+    return out

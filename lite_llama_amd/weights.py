@@ -41,9 +41,12 @@ class Region:
     expert: int | None = None   # index into a stacked [E, ...] parameter
     part: int | None = None     # row block `part` of `parts` equal blocks (of the expert's slice if `expert` is set)
     parts: int = 2
+    rows: tuple[int, int] | None = None   # (first row, count): one member of a projection fused from UNEQUAL members
 
     def __call__(self, param: torch.Tensor) -> torch.Tensor:
         view = param if self.expert is None else param[self.expert]
+        if self.rows is not None:
+            return view.narrow(0, self.rows[0], self.rows[1])
         if self.part is not None:
             rows = view.shape[0] // self.parts
             view = view.narrow(0, self.part * rows, rows)
@@ -529,8 +532,66 @@ def quantization_from_hf_config(config: Mapping):
     raise ValueError(f"unsupported quant_method {method!r}; supported: awq, fp8, gptq")
 
 
+# ------------------------------------------------------------------------------------- #
+# model families: config.json -> which model class, geometry reader and key translation
+# ------------------------------------------------------------------------------------- #
+def model_family(config: Mapping) -> str:
+    """The family name a ``config.json`` asks for: HuggingFace checkpoints say ``model_type``; layered models
+    (model_layers.py) say ``architecture``."""
+    if "architecture" in config and "model_type" not in config:
+        return str(config["architecture"]).lower()
+    return str(config.get("model_type", "")).lower()
+
+
+def _layered_translator(geo) -> Translator:
+    """Tensor names of a layered checkpoint (``l<i>.mix.q``, ``l<i>.mlp.up``, ``loop.in``, ...) -> parameters of
+    :class:`lite_llama_amd.model_layers.LayeredLM`; the members of a fused projection land in their row ranges."""
+    fixed = {"embed": "embed_tokens.weight", "loop.in": "loop_in.weight", "loop.step": "loop_step",
+             "final.norm": "norm_weight", "head": "lm_head.weight"}
+    per_layer = {"norm1": "norm1_weight", "norm2": "norm2_weight", "shift": "shift", "mix.o": "mixer.o_proj.weight",
+                 "mlp.up": "mlp.up_proj.weight", "mlp.down": "mlp.down_proj.weight", "mlp.act": "mlp.act"}
+    by_kind = {"hgrn2": {"mix.f.b": "mixer.f_bias", "mix.lower": "mixer.lower", "mix.norm": "mixer.out_norm_weight"},
+               "attention": {"mix.q.norm": "mixer.q_norm_weight", "mix.k.norm": "mixer.k_norm_weight", "mix.sink": "mixer.sink"}}
+
+    def fused(spec):
+        qk, v = spec.heads * spec.dim, spec.heads * spec.vdim
+        if spec.kind == "hgrn2":
+            return "mixer.qfv_proj.weight", {"mix.q": (0, qk), "mix.f": (qk, qk), "mix.v": (2 * qk, v)}
+        k, v = spec.kv_heads * spec.dim, spec.kv_heads * spec.vdim
+        return "mixer.qkv_proj.weight", {"mix.q": (0, qk), "mix.k": (qk, k), "mix.v": (qk + k, v)}
+
+    def translate(key: str) -> Target:
+        if key in fixed:
+            return fixed[key], whole
+        m = re.match(r"^l(\d+)\.(.+)$", key)
+        if m is None or int(m.group(1)) >= len(geo.layers):
+            return key, whole  # unknown: load_weights reports it
+        index, leaf = int(m.group(1)), m.group(2)
+        spec = geo.layers[index].mixer
+        name, members = fused(spec)
+        if leaf in members:
+            return f"layers.{index}.{name}", Region(rows=members[leaf])
+        leaf = by_kind[spec.kind].get(leaf) or per_layer.get(leaf) or leaf
+        return f"layers.{index}.{leaf}", whole
+
+    return translate
+
+
+def _load_layered(config: Mapping, checkpoints_dir, device, dtype=None, **_):
+    from .model_layers import LayeredGeometry, LayeredLM
+
+    geo = LayeredGeometry.from_config(config, name=model_family(config))
+    model = LayeredLM(geo, dtype=dtype or torch.bfloat16).to(device)
+    with torch.no_grad():
+        load_weights(model, hf_weights_iterator(checkpoints_dir, device), _layered_translator(geo))
+    return model.eval()
+
+
+MODEL_FAMILIES: dict[str, Callable] = {"rakevik": _load_layered}
+
+
 def load_pretrained(checkpoints_dir: str | Path, *, device: str | torch.device = "cuda", quantization: str | None = None,
-                    compact: bool = True):
+                    compact: bool = True, dtype=None):
     """Build the model a checkpoint directory describes and fill it (executor/loader.py:104-147): ``config.json`` ->
     geometry + weight format, parameters allocated on ``device``, checkpoint streamed in (this rank's shards),
     optional load-time quantisation (``quantization``: a ``--quantization`` scheme name) of an fp16 checkpoint.
@@ -545,6 +606,11 @@ def load_pretrained(checkpoints_dir: str | Path, *, device: str | torch.device =
 
     with open(Path(checkpoints_dir) / "config.json") as f:
         config = json.load(f)
+    family = MODEL_FAMILIES.get(model_family(config))
+    if family is not None:
+        if quantization:
+            raise ValueError(f"--quantization is not available for the {model_family(config)} family")
+        return family(config, checkpoints_dir, device, dtype=dtype)
     quant, int4 = quantization_from_hf_config(config)
     model = CausalLM(geometry_from_hf_config(config), quant)
     runtime = QuantConfig.for_runtime_scheme(quantization) if quantization and quant is None and int4 is None else None
