@@ -20,13 +20,16 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "liblite_llama_amd.so"
 ARCH = "gfx950"
-FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off",
-         # no packed fp32 arithmetic from ordinary float code (the host pass warns that it does not know the feature)
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off"]
 FLAGS += os.environ.get("LL_EXTRA_HIPCC_FLAGS", "").split()  # debug builds (e.g. -DV2_DEBUG_ABLATE)
 # per-source flags.  gemm_short.hip: its kernel's first 16 argument dwords arrive in SGPRs with the wave (gfx950 kernarg preload)
 # instead of through dependent scalar loads -- a launch of ~5 us spends ~0.3 us there otherwise.
-FILE_FLAGS = {"gemm_short.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"]}
+# seq_mix.hip / ragged_attn.hip: no packed fp32 arithmetic made from ordinary float code (the host pass warns that it does not
+# know the feature).  The older sources keep the flags their bit-exactness tests were pinned under: with the feature off, two
+# norm kernels that must agree bit for bit (rows summed over MoE slots vs. summed first) select different roundings.
+_NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+FILE_FLAGS = {"gemm_short.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+              "seq_mix.hip": _NO_PACKED_FP32, "ragged_attn.hip": _NO_PACKED_FP32}
 
 
 # part libraries: the sources ONE model family needs (a fresh checkout serving only that family builds nothing else)
@@ -91,12 +94,17 @@ def build(force: bool = False, verbose: bool = True, part: str | None = None) ->
 
     def compile_one(src: str) -> str:
         obj = os.path.join(objdir, os.path.basename(src)[:-4] + ".o")
+        one = _digest([src]) + " " + " ".join(flags_for(src))  # (covers the headers too)
+        if not force and os.path.exists(obj) and os.path.exists(obj + ".stamp") and open(obj + ".stamp").read() == one:
+            return obj  # an object of exactly this source, headers and flags is there
         cmd = [hipcc, *flags_for(src), "-c", src, "-o", obj]
         if verbose:
             print("[build]", " ".join(cmd), flush=True)
         done = subprocess.run(cmd, stderr=None if verbose else subprocess.PIPE, text=True)
         if done.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{done.stderr or ''}")
+        with open(obj + ".stamp", "w") as f:
+            f.write(one)
         return obj
 
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:

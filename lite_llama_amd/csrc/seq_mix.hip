@@ -330,7 +330,7 @@ extern "C" int ll_residual_set(float* x, const void* y, const void* bias, int64_
 extern "C" int ll_gated_linear_scan_supported(int64_t dk, int64_t dv) {
   if (dk < 1 || dv < 1 || dv > 256) return 0;
   const int64_t kg = 256 / dv < dk ? 256 / dv : dk;
-  return (dk + kg - 1) / kg <= 64 ? 1 : 0;
+  return (dk + kg - 1) / kg <= 128 ? 1 : 0;
 }
 
 extern "C" int ll_gated_linear_scan(const void* q, const void* f, const void* v, int64_t ld, const void* f_bias, const void* lower,
@@ -355,7 +355,8 @@ extern "C" int ll_gated_linear_scan(const void* q, const void* f, const void* v,
   if (rmax <= 4) CALL_R(DT, 4);        \
   else if (rmax <= 16) CALL_R(DT, 16); \
   else if (rmax <= 32) CALL_R(DT, 32); \
-  else CALL_R(DT, 64)
+  else if (rmax <= 64) CALL_R(DT, 64); \
+  else CALL_R(DT, 128)
   LL_BY_DTYPE(dtype, CALL);
 #undef CALL
 #undef CALL_R

@@ -33,7 +33,7 @@ def gated_linear_scan(qfv: torch.Tensor, heads: int, dk: int, dv: int, f_bias, l
     if step.num_tokens != n:
         raise ValueError("gated_linear_scan: the step describes another number of tokens")
     if not gated_linear_scan_supported(dk, dv):
-        raise ValueError(f"gated_linear_scan: head geometry {dk} x {dv} is not served (dv <= 256, <= 64 state rows per thread)")
+        raise ValueError(f"gated_linear_scan: head geometry {dk} x {dv} is not served (dv <= 256, <= 128 state rows per thread)")
     out = torch.empty(n, heads * dv, dtype=dt, device=qfv.device)
     es = qfv.element_size()
     base = qfv.data_ptr()
