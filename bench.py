@@ -91,6 +91,10 @@ def parse():
                          "dense projections' launch list eagerly a few times and exit: the workload of a rocprofv3 --pmc pass")
     ap.add_argument("--no-live-pmc", action="store_true",
                     help="skip the live rocprofv3 --pmc passes (roofline.traffic / mfma_util then carry the stored profile values)")
+    ap.add_argument("--layered", action="store_true",
+                    help="instead of the headline: prefill / decode throughput and per-kernel roofline fractions of the layered "
+                         "family (model_layers.py) beside the closest llama-shaped model at equal sizes (benchmarks/layered_bench.py)")
+    ap.add_argument("--layered-dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--no-reference-order", action="store_true",
                     help="skip the bounded drop-in-route entry (\"reference_order\") of the default N = 1 int4 line")
     return ap.parse_args()
@@ -914,6 +918,11 @@ def main():
             args.no_prefill = True
     if args.as_pmc_probe:
         pmc_probe(args)
+        return
+    if args.layered:
+        from benchmarks.layered_bench import run as layered_run
+
+        print(json.dumps(layered_run(args.layered_dtype)))
         return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         raise SystemExit(self_launch(args))
