@@ -61,7 +61,8 @@ def kernel_table(dev, dtype, width, heads, kv_heads, hd, ff, prefill=(8, 512), d
                           tok_pos=vec([first + j for _ in range(batch) for j in range(count)]),
                           select=vec([i * (first + count) + first + j for i in range(batch) for j in range(count)]),
                           seq_start=vec([i * count for i in range(batch + 1)]), seq_first_pos=vec([first] * batch),
-                          seq_slot=vec(list(range(batch))), seq_parity=vec([0] * batch))
+                          seq_slot=vec(list(range(batch))), seq_parity=vec([0] * batch), longest_run=count,
+                          longest_context=first + count)
 
     for phase, (batch, length) in (("prefill", prefill), ("decode", decode)):
         first, count = (0, length) if phase == "prefill" else (length - 1, 1)

@@ -576,12 +576,14 @@ int ll_cast_pair(void* out, const float* a, const void* a_delta, const float* b,
 int ll_residual_set(float* x, const void* y, const void* bias, int64_t n, int64_t width, int dtype, void* stream);
 /* Gated linear recurrence per (sequence, head): f = lower + (1 - lower) sigmoid(f_raw + f_bias), S <- diag(f) S + (1 - f) v^T,
  * o = S^T silu(q_raw), out = o / sqrt(mean_dv(o^2) + eps) * norm_w.  q, f [n, >= heads dk], v [n, >= heads dv] share the
- * row stride ld; state [slots][heads][dk][dv] fp32 (read when seq_first_pos > 0, written at the end of the run). */
+ * row stride ld; state [slots][heads][dk][dv] fp32 (read when seq_first_pos > 0, written at the end of the run).  n = tokens
+ * of the step; with scratch (fp32, n * heads * dv floats) and longest_run > 2 (most tokens a sequence brings) the wide form
+ * runs: a workgroup per 16 state columns, o through scratch, the output norm as a second launch. */
 int ll_gated_linear_scan_supported(int64_t dk, int64_t dv);
 int ll_gated_linear_scan(const void* q, const void* f, const void* v, int64_t ld, const void* f_bias, const void* lower,
                          const void* norm_w, float eps, void* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
                          const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, float* state,
-                         int dtype, void* stream);
+                         int64_t n, int64_t longest_run, float* scratch, int dtype, void* stream);
 /* Rows [q (heads dk) | k (kv_heads dk) | v (kv_heads dv)] of stride ld: q and k RMS-normed per head (weights [dk] or NULL),
  * q times 1 + temp_coef ln(floor((pos + 1) / temp_every) + 1); q -> q_out [n, heads, dk]; k, v -> cache rows select[t] of
  * k_cache [rows, kv_heads, dk] / v_cache [rows, kv_heads, dv]. */
@@ -595,6 +597,18 @@ int ll_ragged_attention(const void* q, const void* k_cache, const void* v_cache,
                         int64_t tt_stride, const int32_t* seq_req, const int32_t* tok_seq, const int32_t* tok_pos,
                         const void* sink, float scale, void* out, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk,
                         int64_t dv, int dtype, void* stream);
+/* MFMA form for 16-bit storage dtypes (dk, dv multiples of 8, <= 256).  decode == 0: prompt portions (16 consecutive tokens
+ * of a run per wave; longest_run = most tokens a sequence brings).  decode != 0: every sequence brings one token (n == batch);
+ * the query heads of a key/value head share a wave, the context is cut into partitions of ll_ragged_attention_partition()
+ * keys and partials (fp32, n * heads * max_parts * (2 + dv) floats, max_parts = ceil(longest_context / partition); may be
+ * NULL when max_parts == 1) is merged by a second launch.  Weights enter the second product as two 16-bit parts. */
+int ll_ragged_attention_mfma_supported(int64_t dk, int64_t dv, int dtype);
+int64_t ll_ragged_attention_partition(void);
+int ll_ragged_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int32_t* token_table,
+                             int64_t tt_stride, const int32_t* seq_req, const int32_t* seq_start,
+                             const int32_t* seq_first_pos, const void* sink, float scale, void* out, int64_t n,
+                             int64_t batch, int64_t longest_run, int64_t longest_context, int decode, float* partials,
+                             int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -115,12 +115,15 @@ SIGNATURES = {
     "ll_cast_pair": [P, P, P, P, L, L, I, P],
     "ll_residual_set": [P, P, P, L, L, I, P],
     "ll_gated_linear_scan_supported": [L, L],
-    "ll_gated_linear_scan": [P, P, P, L, P, P, P, F, P, L, L, L, L, P, P, P, P, I, P],
+    "ll_gated_linear_scan": [P, P, P, L, P, P, P, F, P, L, L, L, L, P, P, P, P, L, L, P, I, P],
     "ll_qk_norm_cache": [P, L, P, P, F, F, L, P, P, P, P, P, L, L, L, L, L, I, P],
     "ll_ragged_attention": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, L, I, P],
+    "ll_ragged_attention_mfma_supported": [L, L, I],
+    "ll_ragged_attention_partition": [],
+    "ll_ragged_attention_mfma": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, I, P, L, L, L, L, I, P],
 }
 
-_RETURNS_I64 = {"ll_kv_alloc_scratch_bytes", "ll_tp_oneshot_flag_words", "ll_moe_router_workspace_floats", "ll_moe_align_workspace_ints"}
+_RETURNS_I64 = {"ll_ragged_attention_partition", "ll_kv_alloc_scratch_bytes", "ll_tp_oneshot_flag_words", "ll_moe_router_workspace_floats", "ll_moe_align_workspace_ints"}
 _lib = None
 
 

@@ -24,16 +24,16 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=
 FLAGS += os.environ.get("LL_EXTRA_HIPCC_FLAGS", "").split()  # debug builds (e.g. -DV2_DEBUG_ABLATE)
 # per-source flags.  gemm_short.hip: its kernel's first 16 argument dwords arrive in SGPRs with the wave (gfx950 kernarg preload)
 # instead of through dependent scalar loads -- a launch of ~5 us spends ~0.3 us there otherwise.
-# seq_mix.hip / ragged_attn.hip: no packed fp32 arithmetic made from ordinary float code (the host pass warns that it does not
+# seq_mix.hip / ragged_attn*.hip: no packed fp32 arithmetic made from ordinary float code (the host pass warns that it does not
 # know the feature).  The older sources keep the flags their bit-exactness tests were pinned under: with the feature off, two
 # norm kernels that must agree bit for bit (rows summed over MoE slots vs. summed first) select different roundings.
 _NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 FILE_FLAGS = {"gemm_short.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
-              "seq_mix.hip": _NO_PACKED_FP32, "ragged_attn.hip": _NO_PACKED_FP32}
+              "seq_mix.hip": _NO_PACKED_FP32, "ragged_attn.hip": _NO_PACKED_FP32, "ragged_attn_mfma.hip": _NO_PACKED_FP32}
 
 
 # part libraries: the sources ONE model family needs (a fresh checkout serving only that family builds nothing else)
-PARTS = {"ragged": ["seq_mix.hip", "ragged_attn.hip", "kv_paged.hip", "kv_ops.hip", "sampler.hip"]}
+PARTS = {"ragged": ["seq_mix.hip", "ragged_attn.hip", "ragged_attn_mfma.hip", "kv_paged.hip", "kv_ops.hip", "sampler.hip"]}
 
 
 def flags_for(src: str) -> list[str]:

@@ -120,15 +120,33 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(
 __device__ __forceinline__ float softplus_f32(float v) { return v > 20.f ? v : log1pf(expf(v)); }
 
 // xIELU: z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2
-template <int DT>
+__device__ __forceinline__ float xielu_f32(float v, float ap, float an) {
+  return v > 0.f ? ap * v * v + 0.5f * v : an * (expm1f(v) - v) + 0.5f * v;
+}
+
+// VEC: 16-byte pieces (8 sixteen-bit values / 4 floats) when the count and both pointers allow it
+template <int DT, bool VEC>
 __global__ __launch_bounds__(256) void xielu_kernel(void* __restrict__ y, const void* __restrict__ z, const void* __restrict__ pq,
                                                     int64_t n) {
   const float ap = softplus_f32(ldv<DT>(pq, 0));
   const float an = 0.5f + softplus_f32(ldv<DT>(pq, 1));
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    const float v = ldv<DT>(z, i);
-    const float r = v > 0.f ? ap * v * v + 0.5f * v : an * (expm1f(v) - v) + 0.5f * v;
-    stv<DT>(y, i, r);
+  if constexpr (!VEC) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+      stv<DT>(y, i, xielu_f32(ldv<DT>(z, i), ap, an));
+  } else if constexpr (DT == LL_F32) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n / 4; i += (int64_t)gridDim.x * 256) {
+      f32x4 a = ((const f32x4*)z)[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a[j] = xielu_f32(a[j], ap, an);
+      ((f32x4*)y)[i] = a;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n / 8; i += (int64_t)gridDim.x * 256) {
+      U16x8 a = ((const U16x8*)z)[i];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) a.v[j] = from_f32<DT>(xielu_f32(to_f32<DT>(a.v[j]), ap, an));
+      ((U16x8*)y)[i] = a;
+    }
   }
 }
 
@@ -172,6 +190,13 @@ __global__ __launch_bounds__(256) void residual_set_kernel(float* __restrict__ x
 // --------------------------------------------------------------------------------------------------------------------- //
 constexpr int kScanTB = 8;
 
+// sigmoid of the gate and of silu: libm's exp for fp32 storage, the hardware exp2 / reciprocal (1 ulp each) for 16-bit storage
+template <int DT>
+__device__ __forceinline__ float gate_sigmoid(float v) {
+  if constexpr (DT == LL_F32) return 1.0f / (1.0f + expf(-v));
+  else return ll_sigmoidf(v);
+}
+
 template <int DT, int RMAX>
 __global__ __launch_bounds__(256) void gated_linear_scan_kernel(
     const void* __restrict__ q, const void* __restrict__ f, const void* __restrict__ v, int64_t ld, const void* __restrict__ f_bias,
@@ -205,10 +230,9 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(
       const int64_t at = (int64_t)(base + tt) * ld + head * dk + k;
       const float lo = ldv<DT>(lower, head * dk + k);
       const float raw = ldv<DT>(f, at) + ldv<DT>(f_bias, head * dk + k);
-      const float sig = 1.0f / (1.0f + expf(-raw));
-      sf[i] = lo + (1.0f - lo) * sig;
+      sf[i] = lo + (1.0f - lo) * gate_sigmoid<DT>(raw);
       const float qv = ldv<DT>(q, at);
-      sq[i] = qv / (1.0f + expf(-qv));
+      sq[i] = qv * gate_sigmoid<DT>(qv);
     }
     for (int i = tid; i < nt * dv; i += 256) {
       const int tt = i / dv, cc = i - tt * dv;
@@ -260,6 +284,94 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(
     if (r < rows) st[(int64_t)(g + r * kg) * dv + c] = S[r];
 }
 
+
+// Wide form for runs of many tokens: one workgroup per (sequence, head, 16 columns of the state) -- dv / 16 times the
+// workgroups of the form above and dk / 16 state rows per thread instead of dk dv / 256, which is what a run's serial walk
+// costs per token.  Thread (kg, c): column c of the slice, rows kg, kg + 16, ...  The per-head output norm needs all dv
+// columns: o goes to an fp32 scratch [n, heads dv] and head_rmsnorm_kernel finishes.  The state update is the expression of
+// the form above, so both leave the same state bits.
+template <int DT, int RMAX>
+__global__ __launch_bounds__(256) void gated_linear_scan_wide_kernel(
+    const void* __restrict__ q, const void* __restrict__ f, const void* __restrict__ v, int64_t ld, const void* __restrict__ f_bias,
+    const void* __restrict__ lower, float* __restrict__ o_scratch, int heads, int dk, int dv, int tb,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
+    float* __restrict__ state) {
+  extern __shared__ float lds[];
+  const int b = blockIdx.x, head = blockIdx.y, c0 = blockIdx.z * 16;
+  const int tid = threadIdx.x, col = tid & 15, kg = tid >> 4;
+  const bool active = c0 + col < dv && kg < dk;
+  const int rows = kg < dk ? (dk - kg + 15) / 16 : 0;
+  float* sf = lds;                 // [tb][dk] forget gates
+  float* su = sf + tb * dk;        // [tb][dk] 1 - gate
+  float* sq = su + tb * dk;        // [tb][dk] queries
+  float* sv = sq + tb * dk;        // [tb][16] values of the slice
+  float* sp = sv + tb * 16;        // [tb][16 groups][16] partial outputs
+  const int t0 = seq_start[b], t1 = seq_start[b + 1];
+  float* st = state + ((int64_t)seq_slot[b] * heads + head) * dk * dv + c0 + col;
+  const bool carry = seq_first_pos[b] > 0;
+  float S[RMAX];
+#pragma unroll
+  for (int r = 0; r < RMAX; ++r) S[r] = (active && r < rows && carry) ? st[(int64_t)(kg + 16 * r) * dv] : 0.f;
+  for (int base = t0; base < t1; base += tb) {
+    const int nt = t1 - base < tb ? t1 - base : tb;
+    __syncthreads();
+    for (int i = tid; i < nt * dk; i += 256) {
+      const int tt = i / dk, k = i - tt * dk;
+      const int64_t at = (int64_t)(base + tt) * ld + head * dk + k;
+      const float lo = ldv<DT>(lower, head * dk + k);
+      const float fg = lo + (1.0f - lo) * gate_sigmoid<DT>(ldv<DT>(f, at) + ldv<DT>(f_bias, head * dk + k));
+      sf[i] = fg;
+      su[i] = 1.0f - fg;
+      const float qv = ldv<DT>(q, at);
+      sq[i] = qv * gate_sigmoid<DT>(qv);
+    }
+    for (int i = tid; i < nt * 16; i += 256) {
+      const int tt = i >> 4, cc = i & 15;
+      sv[i] = c0 + cc < dv ? ldv<DT>(v, (int64_t)(base + tt) * ld + head * dv + c0 + cc) : 0.f;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float val = sv[tt * 16 + col];
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r) {
+        if (r < rows) {
+          const int k = tt * dk + kg + 16 * r;
+          S[r] = sf[k] * S[r] + su[k] * val;
+          acc += S[r] * sq[k];
+        }
+      }
+      sp[(tt * 16 + kg) * 16 + col] = acc;
+    }
+    __syncthreads();
+    for (int i = tid; i < nt * 16; i += 256) {
+      const int tt = i >> 4, cc = i & 15;
+      float o = 0.f;
+#pragma unroll
+      for (int g2 = 0; g2 < 16; ++g2) o += sp[(tt * 16 + g2) * 16 + cc];
+      if (c0 + cc < dv) o_scratch[((int64_t)(base + tt) * heads + head) * dv + c0 + cc] = o;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RMAX; ++r)
+    if (active && r < rows) st[(int64_t)(kg + 16 * r) * dv] = S[r];
+}
+
+// one wave per (token, head): out = o / sqrt(mean_dv(o^2) + eps) * w
+template <int DT>
+__global__ __launch_bounds__(256) void head_rmsnorm_kernel(void* __restrict__ out, const float* __restrict__ o,
+                                                           const void* __restrict__ w, float eps, int64_t items, int dv) {
+  const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= items) return;
+  const int lane = threadIdx.x & 63;
+  const float* src = o + item * dv;
+  float ss = 0.f;
+  for (int cc = lane; cc < dv; cc += 64) ss += src[cc] * src[cc];
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
+  for (int cc = lane; cc < dv; cc += 64) stv<DT>(out, item * dv + cc, src[cc] * inv * ldv<DT>(w, cc));
+}
+
 inline unsigned flat_grid(int64_t total) {
   const int64_t g = (total + 255) / 256;
   return (unsigned)(g < 1 ? 1 : (g > 16384 ? 16384 : g));
@@ -298,7 +410,11 @@ extern "C" int ll_xielu(void* y, const void* z, const void* pq, int64_t n, int d
   if (n < 0) return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
   if (!y || !z || !pq) return LL_ERR_ARG;
-#define CALL(DT) xielu_kernel<DT><<<dim3(flat_grid(n)), 256, 0, (hipStream_t)stream>>>(y, z, pq, n)
+  const int per = dtype == LL_F32 ? 4 : 8;
+  const bool vec = n % per == 0 && ll_aligned16(y) && ll_aligned16(z);
+#define CALL(DT)                                                                                           \
+  if (vec) xielu_kernel<DT, true><<<dim3(flat_grid(n / per)), 256, 0, (hipStream_t)stream>>>(y, z, pq, n); \
+  else xielu_kernel<DT, false><<<dim3(flat_grid(n)), 256, 0, (hipStream_t)stream>>>(y, z, pq, n)
   LL_BY_DTYPE(dtype, CALL);
 #undef CALL
   return LL_LAUNCH_CHECK();
@@ -336,18 +452,40 @@ extern "C" int ll_gated_linear_scan_supported(int64_t dk, int64_t dv) {
 extern "C" int ll_gated_linear_scan(const void* q, const void* f, const void* v, int64_t ld, const void* f_bias, const void* lower,
                                     const void* norm_w, float eps, void* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
                                     const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, float* state,
-                                    int dtype, void* stream) {
+                                    int64_t n, int64_t longest_run, float* scratch, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
-  if (batch < 0 || heads < 1 || heads > 65535 || !ll_gated_linear_scan_supported(dk, dv)) return LL_ERR_SHAPE;
+  if (batch < 0 || n < 0 || heads < 1 || heads > 65535 || !ll_gated_linear_scan_supported(dk, dv)) return LL_ERR_SHAPE;
   if (batch == 0) return LL_OK;
   if (!q || !f || !v || !f_bias || !lower || !norm_w || !out || !seq_start || !seq_first_pos || !seq_slot || !state)
     return LL_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  if (scratch && longest_run > 2 && dk <= 256) {
+    // wide form + output norm (runs of several tokens: prompt portions, mixed steps)
+    const int tb = dk <= 128 ? 16 : 8;
+    const size_t lds = sizeof(float) * (size_t)(tb * (3 * dk + 16 + 256));
+    const dim3 grid((unsigned)batch, (unsigned)heads, (unsigned)((dv + 15) / 16));
+    const int rmax = (int)((dk + 15) / 16);
+#define CALL_W(DT, R)                                                                                                          \
+  gated_linear_scan_wide_kernel<DT, R><<<grid, 256, lds, st>>>(q, f, v, ld, f_bias, lower, scratch, (int)heads, (int)dk, (int)dv, \
+                                                               tb, seq_start, seq_first_pos, seq_slot, state)
+#define CALL(DT)                     \
+  if (rmax <= 4) CALL_W(DT, 4);      \
+  else if (rmax <= 8) CALL_W(DT, 8); \
+  else CALL_W(DT, 16)
+    LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+#undef CALL_W
+    const int64_t items = n * heads;
+#define CALL(DT) head_rmsnorm_kernel<DT><<<dim3((unsigned)((items + 3) / 4)), 256, 0, st>>>(out, scratch, norm_w, eps, items, (int)dv)
+    LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return LL_LAUNCH_CHECK();
+  }
   const int kg = (int)(256 / dv < dk ? 256 / dv : dk);
   const int rmax = (int)((dk + kg - 1) / kg);
   const size_t lds = sizeof(float) * (size_t)(kScanTB * (2 * dk + dv) + kScanTB * kg * dv + kScanTB * dv + kScanTB);
   if (lds > 64 * 1024) return LL_ERR_SHAPE;
   const dim3 grid((unsigned)batch, (unsigned)heads);
-  hipStream_t st = (hipStream_t)stream;
 #define CALL_R(DT, R)                                                                                                        \
   gated_linear_scan_kernel<DT, R><<<grid, 256, lds, st>>>(q, f, v, ld, f_bias, lower, norm_w, eps, out, (int)heads, (int)dk, \
                                                           (int)dv, seq_start, seq_first_pos, seq_slot, state)

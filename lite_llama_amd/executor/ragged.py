@@ -34,6 +34,8 @@ class RaggedStep:
     seq_first_pos: torch.Tensor
     seq_slot: torch.Tensor
     seq_parity: torch.Tensor
+    longest_run: int = 0       # most tokens a sequence brings (host copy; 0: not known)
+    longest_context: int = 0   # longest sequence after this step (host copy; 0: not known)
 
     @property
     def seq_req(self) -> torch.Tensor:
@@ -133,7 +135,7 @@ class RaggedRunner:
         select = rows.reshape(-1)[torch.tensor(pick, dtype=torch.long, device=dev)].contiguous()
         step = RaggedStep(num_tokens=len(tokens), num_seqs=len(entries), tok_seq=vec(tok_seq), tok_pos=vec(tok_pos), select=select,
                           seq_start=vec(starts), seq_first_pos=vec(first), seq_slot=seq_slot,
-                          seq_parity=vec([self._parity[s] for s in slots]))
+                          seq_parity=vec([self._parity[s] for s in slots]), longest_run=longest, longest_context=max(new_len))
         for s, n in zip(slots, new_len):
             self._len[s] = n
             self._parity[s] ^= 1

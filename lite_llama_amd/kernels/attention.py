@@ -3,6 +3,8 @@ and flashattention2_nopad.py:175-231 over the HIP C-ABI."""
 
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .. import _lib as L
@@ -326,6 +328,19 @@ def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=
     if step.num_tokens != n:
         raise ValueError("ragged_attention: the step describes another number of tokens")
     out = torch.empty(n, heads * dv, dtype=dt, device=q.device)
+    if (step.longest_run and step.longest_context and L.has("ll_ragged_attention_mfma") and not os.environ.get("LL_RAGGED_ATTN_VALU")
+            and L.lib().ll_ragged_attention_mfma_supported(dk, dv, L.dtype_code(dt))):
+        # 16-bit storage: the MFMA form -- tokens of a run as the columns of a wave (prompt portions, mixed steps), or, when every
+        # sequence brings one decoded token, the query heads of a key/value head, with the context cut into partitions
+        decode = step.longest_run == 1
+        parts = -(-step.longest_context // int(L.lib().ll_ragged_attention_partition())) if decode else 1
+        scratch = torch.empty(n * heads * parts * (2 + dv), dtype=torch.float32, device=q.device) if parts > 1 else None
+        L.check(L.lib().ll_ragged_attention_mfma(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), token_table.data_ptr(), token_table.stride(0),
+            step.seq_req.data_ptr(), step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(), L.ptr(sink), float(scale),
+            out.data_ptr(), n, step.num_seqs, step.longest_run, step.longest_context, 1 if decode else 0, L.ptr(scratch), heads,
+            kv_heads, dk, dv, L.dtype_code(dt), L.stream_ptr()), "ragged_attention_mfma")
+        return out
     L.check(L.lib().ll_ragged_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), token_table.data_ptr(),
                                         token_table.stride(0), step.seq_req.data_ptr(), step.tok_seq.data_ptr(),
                                         step.tok_pos.data_ptr(), L.ptr(sink), float(scale), out.data_ptr(), n, heads, kv_heads, dk,

@@ -35,11 +35,14 @@ def gated_linear_scan(qfv: torch.Tensor, heads: int, dk: int, dv: int, f_bias, l
     if not gated_linear_scan_supported(dk, dv):
         raise ValueError(f"gated_linear_scan: head geometry {dk} x {dv} is not served (dv <= 256, <= 128 state rows per thread)")
     out = torch.empty(n, heads * dv, dtype=dt, device=qfv.device)
+    # runs of several tokens take the wide form (a workgroup per 16 state columns; o through an fp32 scratch, then the norm)
+    scratch = torch.empty(n, heads * dv, dtype=torch.float32, device=qfv.device) if step.longest_run > 2 and dk <= 256 else None
     es = qfv.element_size()
     base = qfv.data_ptr()
     L.check(L.lib().ll_gated_linear_scan(
         base, base + heads * dk * es, base + 2 * heads * dk * es, qfv.stride(0), f_bias.data_ptr(), lower.data_ptr(),
         norm_weight.data_ptr(), float(eps), out.data_ptr(), step.num_seqs, heads, dk, dv, step.seq_start.data_ptr(),
-        step.seq_first_pos.data_ptr(), step.seq_slot.data_ptr(), state.data_ptr(), L.dtype_code(dt), L.stream_ptr()),
+        step.seq_first_pos.data_ptr(), step.seq_slot.data_ptr(), state.data_ptr(), n, step.longest_run, L.ptr(scratch),
+        L.dtype_code(dt), L.stream_ptr()),
         "gated_linear_scan")
     return out

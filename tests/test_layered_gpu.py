@@ -36,7 +36,8 @@ def _step(seqs, table=None):
 
     return RaggedStep(num_tokens=starts[-1], num_seqs=len(seqs), tok_seq=vec(tok_seq), tok_pos=vec(tok_pos), select=vec(select),
                       seq_start=vec(starts), seq_first_pos=vec([s[1] for s in seqs]), seq_slot=vec([s[0] for s in seqs]),
-                      seq_parity=vec([s[3] for s in seqs]))
+                      seq_parity=vec([s[3] for s in seqs]), longest_run=max(s[2] for s in seqs),
+                      longest_context=max(s[1] + s[2] for s in seqs))
 
 
 def _close(got, want, tol):
@@ -200,8 +201,9 @@ def test_sink_attention_portions_decode_and_a_neighbour_in_the_batch(dtype, head
     _close(got, want, 5e-5 if dtype == torch.float32 else 2e-2)
 
 
-@pytest.mark.parametrize("far", [0, 3, 63, 64, 127, 128, 600])
-def test_one_far_key_among_hundreds_is_found(far):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("far", [0, 3, 63, 64, 127, 128, 255, 256, 600])
+def test_one_far_key_among_hundreds_is_found(far, dtype):
     """Query and key of one far position are made parallel and the scale sharp: the output must be that position's value,
     from a prompt portion and from a decoded token alike."""
     heads, kv_heads, dk, dv, T_len = 2, 1, 16, 8, 700
@@ -214,12 +216,12 @@ def test_one_far_key_among_hundreds_is_found(far):
     plan = [[(1, 0, 64)], [(1, 64, T_len - 65)], [(1, T_len - 1, 1)]]   # the last token is decoded alone
     ones = torch.ones(dk)
     sink = torch.tensor([-30.0, 0.5])
-    got, want = _attention_case(torch.float32, heads, kv_heads, dk, dv, T_len, plan, temp=(0.0, 1), scale=4.0, qkv_rows=rows,
-                                sink=sink)
-    _close(got, want, 5e-5)
-    v_far = rows[far, (heads + kv_heads) * dk:]
+    sharp = 4.0 if dtype == torch.float32 else 1.0   # (16-bit queries and keys: a score of 36 +- 0.1 instead of 144 +- 0.5)
+    got, want = _attention_case(dtype, heads, kv_heads, dk, dv, T_len, plan, temp=(0.0, 1), scale=sharp, qkv_rows=rows, sink=sink)
+    _close(got, want, 5e-5 if dtype == torch.float32 else 3e-2)
+    v_far = rows[far, (heads + kv_heads) * dk:].to(dtype)
     for t in (T_len - 1, T_len - 2):
-        _close(got[t, :dv], v_far, 1e-3)
+        _close(got[t, :dv], v_far.float(), 1e-3 if dtype == torch.float32 else 1e-2)
 
 
 def test_sink_takes_its_share_of_the_softmax():
@@ -233,6 +235,18 @@ def test_sink_takes_its_share_of_the_softmax():
     mid, want_mid = _attention_case(torch.float32, heads, kv_heads, dk, dv, 20, plan, sink=torch.tensor([0.0, 0.0]))
     _close(mid, want_mid, 5e-5)
     assert (mid[0].abs() < want_hi[0, dv:].abs().max() + 10).all() and not torch.allclose(mid[:, dv:].cpu(), hi[:, dv:].cpu())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,dk,dv", [(20, 1, 32, 16), (4, 2, 128, 128), (2, 1, 200, 72)])
+def test_decoded_tokens_over_several_partitions_of_the_context(dtype, heads, kv_heads, dk, dv):
+    """Contexts of 250 .. 530 tokens: decoded tokens see one, two and three partitions (cut every 256 keys), a group of 20
+    query heads needs two column tiles; a neighbour with a short context rides along."""
+    T_len = 530
+    plan = [[(1, 0, 250), (0, 0, 3)]] + [[(1, 250 + i, 1), (0, 3 + i, 1)] for i in range(10)] + [[(1, 260, 250)]] + \
+           [[(1, 510 + i, 1), (0, 13 + i, 1)] for i in range(20)]
+    got, want = _attention_case(dtype, heads, kv_heads, dk, dv, T_len, plan, temp=(0.3, 128))
+    _close(got, want, 5e-5 if dtype == torch.float32 else 2e-2)
 
 
 @pytest.mark.parametrize("every", [1, 3, 64])
