@@ -83,7 +83,8 @@ def kernel_table(dev, dtype, width, heads, kv_heads, hd, ff, prefill=(8, 512), d
         z = torch.randn(n, ff, device=dev).to(dtype)
         pq = torch.tensor([0.3, -0.2], device=dev).to(dtype)
         t_new = _time(lambda: xielu(z, pq))
-        t_old = _time(lambda: swiglu_forward(z, z))
+        z2 = torch.randn(n, ff, device=dev).to(dtype)
+        t_old = _time(lambda: swiglu_forward(z, z2))
         like = _entry("swiglu_forward", t_old, n * ff * es * 3, 0)
         out.append(dict(_entry("xielu", t_new, n * ff * es * 2, 0, like), phase=phase))
         # attention

@@ -120,8 +120,15 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(
 __device__ __forceinline__ float softplus_f32(float v) { return v > 20.f ? v : log1pf(expf(v)); }
 
 // xIELU: z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2
+// (16-bit storage: exp(v) - 1 through the hardware exp2 -- its absolute error of ~1e-7 sits under the z / 2 term by more than the
+// storage format resolves; fp32 storage: libm's expm1)
+template <int DT>
 __device__ __forceinline__ float xielu_f32(float v, float ap, float an) {
-  return v > 0.f ? ap * v * v + 0.5f * v : an * (expm1f(v) - v) + 0.5f * v;
+  if (v > 0.f) return ap * v * v + 0.5f * v;
+  float em1;
+  if constexpr (DT == LL_F32) em1 = expm1f(v);
+  else em1 = __builtin_amdgcn_exp2f(v * 1.44269504088896341f) - 1.0f;
+  return an * (em1 - v) + 0.5f * v;
 }
 
 // VEC: 16-byte pieces (8 sixteen-bit values / 4 floats) when the count and both pointers allow it
@@ -132,19 +139,19 @@ __global__ __launch_bounds__(256) void xielu_kernel(void* __restrict__ y, const 
   const float an = 0.5f + softplus_f32(ldv<DT>(pq, 1));
   if constexpr (!VEC) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
-      stv<DT>(y, i, xielu_f32(ldv<DT>(z, i), ap, an));
+      stv<DT>(y, i, xielu_f32<DT>(ldv<DT>(z, i), ap, an));
   } else if constexpr (DT == LL_F32) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n / 4; i += (int64_t)gridDim.x * 256) {
       f32x4 a = ((const f32x4*)z)[i];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) a[j] = xielu_f32(a[j], ap, an);
+      for (int j = 0; j < 4; ++j) a[j] = xielu_f32<DT>(a[j], ap, an);
       ((f32x4*)y)[i] = a;
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n / 8; i += (int64_t)gridDim.x * 256) {
       U16x8 a = ((const U16x8*)z)[i];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) a.v[j] = from_f32<DT>(xielu_f32(to_f32<DT>(a.v[j]), ap, an));
+      for (int j = 0; j < 8; ++j) a.v[j] = from_f32<DT>(xielu_f32<DT>(to_f32<DT>(a.v[j]), ap, an));
       ((U16x8*)y)[i] = a;
     }
   }

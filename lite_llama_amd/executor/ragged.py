@@ -125,21 +125,23 @@ class RaggedRunner:
             tok_pos += range(f, f + c)
             pick += range(i * longest + longest - c, (i + 1) * longest)
             tokens += [int(t) for t in toks]
-        dev = self.device
-
-        def vec(values):
-            return torch.tensor(values, dtype=torch.int32, device=dev)
-
-        seq_slot = vec(slots)
-        rows = self.cache.extend(seq_slot, vec(new_len), longest, self.token_table)
-        select = rows.reshape(-1)[torch.tensor(pick, dtype=torch.long, device=dev)].contiguous()
-        step = RaggedStep(num_tokens=len(tokens), num_seqs=len(entries), tok_seq=vec(tok_seq), tok_pos=vec(tok_pos), select=select,
-                          seq_start=vec(starts), seq_first_pos=vec(first), seq_slot=seq_slot,
-                          seq_parity=vec([self._parity[s] for s in slots]), longest_run=longest, longest_context=max(new_len))
+        # every vector of the step crosses to the device in ONE copy: a packed int32 tensor, sliced into views
+        parts = [tok_seq, tok_pos, starts, first, slots, [self._parity[s] for s in slots], new_len, pick, tokens]
+        packed = torch.tensor([v for part in parts for v in part], dtype=torch.int32).to(self.device, non_blocking=True)
+        views, at = [], 0
+        for part in parts:
+            views.append(packed[at:at + len(part)])
+            at += len(part)
+        v_tok_seq, v_tok_pos, v_starts, v_first, v_slots, v_parity, v_new_len, v_pick, v_tokens = views
+        rows = self.cache.extend(v_slots, v_new_len, longest, self.token_table)
+        select = rows.reshape(-1)[v_pick].contiguous()
+        step = RaggedStep(num_tokens=len(tokens), num_seqs=len(entries), tok_seq=v_tok_seq, tok_pos=v_tok_pos, select=select,
+                          seq_start=v_starts, seq_first_pos=v_first, seq_slot=v_slots, seq_parity=v_parity, longest_run=longest,
+                          longest_context=max(new_len))
         for s, n in zip(slots, new_len):
             self._len[s] = n
             self._parity[s] ^= 1
-        return step, torch.tensor(tokens, dtype=torch.long, device=dev)
+        return step, v_tokens
 
     @torch.no_grad()
     def step(self, entries: Sequence[tuple[int, Sequence[int]]], logits_rows: Sequence[int] | None = None, *,
@@ -149,7 +151,10 @@ class RaggedRunner:
         ``[rows, vocab]`` logits in the model's dtype, or ``None``."""
         step, token_ids = self.build_step(entries)
         if logits_rows is None:
-            logits_rows = [int(v) - 1 for v in step.seq_start.tolist()[1:]]
+            logits_rows, at = [], 0
+            for _, toks in entries:
+                at += len(toks)
+                logits_rows.append(at - 1)
         rows = torch.tensor(list(logits_rows), dtype=torch.long, device=self.device) if len(logits_rows) else None
         out = self.model(token_ids, step, self.cache, self.token_table, logits_rows=rows, collect_layers=collect_layers)
         return out
