@@ -577,8 +577,9 @@ int ll_residual_set(float* x, const void* y, const void* bias, int64_t n, int64_
 /* Gated linear recurrence per (sequence, head): f = lower + (1 - lower) sigmoid(f_raw + f_bias), S <- diag(f) S + (1 - f) v^T,
  * o = S^T silu(q_raw), out = o / sqrt(mean_dv(o^2) + eps) * norm_w.  q, f [n, >= heads dk], v [n, >= heads dv] share the
  * row stride ld; state [slots][heads][dk][dv] fp32 (read when seq_first_pos > 0, written at the end of the run).  n = tokens
- * of the step; with scratch (fp32, n * heads * dv floats) and longest_run > 2 (most tokens a sequence brings) the wide form
- * runs: a workgroup per 16 state columns, o through scratch, the output norm as a second launch. */
+ * of the step; with scratch (fp32, n * heads * dv floats), dk <= 256 and either longest_run > 2 (most tokens a sequence
+ * brings) or fewer than 1024 (sequence, head) pairs, the wide form runs: a workgroup per 16 state columns, o through scratch,
+ * the output norm as a second launch. */
 int ll_gated_linear_scan_supported(int64_t dk, int64_t dv);
 int ll_gated_linear_scan(const void* q, const void* f, const void* v, int64_t ld, const void* f_bias, const void* lower,
                          const void* norm_w, float eps, void* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,

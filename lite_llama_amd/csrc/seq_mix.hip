@@ -117,6 +117,121 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(
   }
 }
 
+
+// Register-cached form of the kernel above for widths <= 4096 that are multiples of 4: every thread keeps its 4-element
+// pieces of the row's sum (and of the previous row's) in registers -- one pass over global memory, 16-byte residual
+// accesses, 8-byte (16-bit storage) activation accesses.  Same arithmetic and the same reduction order as the plain form.
+template <int DT>
+__device__ __forceinline__ f32x4 ld4(const void* p, int64_t i) {  // four storage-dtype values at element i (multiple of 4)
+  if constexpr (DT == LL_F32) {
+    return *reinterpret_cast<const f32x4*>((const float*)p + i);
+  } else {
+    const uint2 u = *reinterpret_cast<const uint2*>((const uint16_t*)p + i);
+    return f32x4{to_f32<DT>((uint16_t)(u.x & 0xffff)), to_f32<DT>((uint16_t)(u.x >> 16)), to_f32<DT>((uint16_t)(u.y & 0xffff)),
+                 to_f32<DT>((uint16_t)(u.y >> 16))};
+  }
+}
+template <int DT>
+__device__ __forceinline__ void st4(void* p, int64_t i, f32x4 v) {
+  if constexpr (DT == LL_F32) {
+    *reinterpret_cast<f32x4*>((float*)p + i) = v;
+  } else {
+    uint2 u;
+    u.x = (uint32_t)from_f32<DT>(v[0]) | ((uint32_t)from_f32<DT>(v[1]) << 16);
+    u.y = (uint32_t)from_f32<DT>(v[2]) | ((uint32_t)from_f32<DT>(v[3]) << 16);
+    *reinterpret_cast<uint2*>((uint16_t*)p + i) = u;
+  }
+}
+
+template <int DT, int NV>
+__global__ __launch_bounds__(256) void add_rmsnorm_shift_vec_kernel(
+    const float* __restrict__ x_in, const void* __restrict__ delta, float* __restrict__ x_out, const void* __restrict__ weight,
+    const void* __restrict__ shift, void* __restrict__ y, int64_t n, int width, float eps, const int32_t* __restrict__ tok_seq,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
+    const int32_t* __restrict__ seq_parity, float* __restrict__ state, int64_t state_half) {
+  __shared__ float red[4];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x;
+  f32x4 s[NV], sp[NV];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = (tid + 256 * j) * 4;
+    s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (i < width) {
+      s[j] = *reinterpret_cast<const f32x4*>(x_in + t * width + i);
+      if (delta) {
+        const f32x4 d = ld4<DT>(delta, t * width + i);
+        s[j][0] += d[0]; s[j][1] += d[1]; s[j][2] += d[2]; s[j][3] += d[3];
+      }
+      // (element order i, i + 1, ..: the plain form adds the same values thread by thread in steps of 256 -- the per-thread
+      // partial sums differ, so the two forms agree to rounding, and each is deterministic on its own)
+      ss += s[j][0] * s[j][0]; ss += s[j][1] * s[j][1]; ss += s[j][2] * s[j][2]; ss += s[j][3] * s[j][3];
+    }
+  }
+  ss = block_sum256(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  int mode = 0, b = 0;
+  const float* prev_state = nullptr;
+  float inv_prev = 0.f;
+  if (shift) {
+    b = tok_seq[t];
+    if (t > seq_start[b]) {
+      mode = 1;
+      float q = 0.f;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int i = (tid + 256 * j) * 4;
+        sp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (i < width) {
+          sp[j] = *reinterpret_cast<const f32x4*>(x_in + (t - 1) * width + i);
+          if (delta) {
+            const f32x4 d = ld4<DT>(delta, (t - 1) * width + i);
+            sp[j][0] += d[0]; sp[j][1] += d[1]; sp[j][2] += d[2]; sp[j][3] += d[3];
+          }
+          q += sp[j][0] * sp[j][0]; q += sp[j][1] * sp[j][1]; q += sp[j][2] * sp[j][2]; q += sp[j][3] * sp[j][3];
+        }
+      }
+      q = block_sum256(q, red);
+      inv_prev = 1.0f / sqrtf(q / (float)width + eps);
+    } else if (seq_first_pos[b] > 0) {
+      mode = 2;
+      prev_state = state + (int64_t)seq_parity[b] * state_half + (int64_t)seq_slot[b] * width;
+    } else {
+      mode = 3;
+    }
+  }
+  float* keep = nullptr;
+  if (shift && t == seq_start[b + 1] - 1)
+    keep = state + (int64_t)(1 - seq_parity[b]) * state_half + (int64_t)seq_slot[b] * width;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = (tid + 256 * j) * 4;
+    if (i < width) {
+      if (delta) *reinterpret_cast<f32x4*>(x_out + t * width + i) = s[j];
+      const f32x4 w = ld4<DT>(weight, i);
+      f32x4 h, o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) h[e] = s[j][e] * inv * w[e];
+      o = h;
+      if (mode) {
+        f32x4 hp = {0.f, 0.f, 0.f, 0.f};
+        if (mode == 1) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) hp[e] = sp[j][e] * inv_prev * w[e];
+        } else if (mode == 2) {
+          hp = *reinterpret_cast<const f32x4*>(prev_state + i);
+        }
+        const f32x4 mu = ld4<DT>(shift, i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = h[e] + (hp[e] - h[e]) * mu[e];
+        if (keep) *reinterpret_cast<f32x4*>(keep + i) = h;
+      }
+      st4<DT>(y, t * width + i, o);
+    }
+  }
+}
+
 __device__ __forceinline__ float softplus_f32(float v) { return v > 20.f ? v : log1pf(expf(v)); }
 
 // xIELU: z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2
@@ -403,12 +518,20 @@ extern "C" int ll_add_rmsnorm_shift(const float* x_in, const void* delta, float*
   if (!x_in || !weight || !y || (delta && !x_out)) return LL_ERR_ARG;
   if (delta && x_out == x_in && shift) return LL_ERR_ARG;  // the previous row is re-read: it must still hold the old sum
   if (shift && (!tok_seq || !seq_start || !seq_first_pos || !seq_slot || !seq_parity || !state)) return LL_ERR_ARG;
-#define CALL(DT)                                                                                                          \
-  add_rmsnorm_shift_kernel<DT><<<dim3((unsigned)n), 256, 0, (hipStream_t)stream>>>(                                         \
-      x_in, delta, x_out, weight, shift, y, n, (int)width, eps, tok_seq, seq_start, seq_first_pos, seq_slot, seq_parity, state, \
-      state_half)
+#define LL_NORM_ARGS \
+  x_in, delta, x_out, weight, shift, y, n, (int)width, eps, tok_seq, seq_start, seq_first_pos, seq_slot, seq_parity, state, state_half
+  const bool vec = width % 4 == 0 && width <= 4096 && ll_aligned16(x_in) && (!delta || (ll_aligned16(delta) && ll_aligned16(x_out))) &&
+                   ll_aligned16(weight) && ll_aligned16(y) && (!shift || (ll_aligned16(shift) && ll_aligned16(state)));
+  const dim3 grid((unsigned)n);
+  hipStream_t st = (hipStream_t)stream;
+#define CALL(DT)                                                                                   \
+  if (!vec) add_rmsnorm_shift_kernel<DT><<<grid, 256, 0, st>>>(LL_NORM_ARGS);                      \
+  else if (width <= 1024) add_rmsnorm_shift_vec_kernel<DT, 1><<<grid, 256, 0, st>>>(LL_NORM_ARGS); \
+  else if (width <= 2048) add_rmsnorm_shift_vec_kernel<DT, 2><<<grid, 256, 0, st>>>(LL_NORM_ARGS); \
+  else add_rmsnorm_shift_vec_kernel<DT, 4><<<grid, 256, 0, st>>>(LL_NORM_ARGS)
   LL_BY_DTYPE(dtype, CALL);
 #undef CALL
+#undef LL_NORM_ARGS
   return LL_LAUNCH_CHECK();
 }
 
@@ -466,8 +589,9 @@ extern "C" int ll_gated_linear_scan(const void* q, const void* f, const void* v,
   if (!q || !f || !v || !f_bias || !lower || !norm_w || !out || !seq_start || !seq_first_pos || !seq_slot || !state)
     return LL_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
-  if (scratch && longest_run > 2 && dk <= 256) {
-    // wide form + output norm (runs of several tokens: prompt portions, mixed steps)
+  if (scratch && dk <= 256 && (longest_run > 2 || batch * heads < 1024)) {
+    // wide form + output norm: runs of several tokens (prompt portions, mixed steps), and decode batches too small to fill the
+    // chip with one workgroup per (sequence, head)
     const int tb = dk <= 128 ? 16 : 8;
     const size_t lds = sizeof(float) * (size_t)(tb * (3 * dk + 16 + 256));
     const dim3 grid((unsigned)batch, (unsigned)heads, (unsigned)((dv + 15) / 16));

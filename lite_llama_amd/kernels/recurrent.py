@@ -35,8 +35,9 @@ def gated_linear_scan(qfv: torch.Tensor, heads: int, dk: int, dv: int, f_bias, l
     if not gated_linear_scan_supported(dk, dv):
         raise ValueError(f"gated_linear_scan: head geometry {dk} x {dv} is not served (dv <= 256, <= 128 state rows per thread)")
     out = torch.empty(n, heads * dv, dtype=dt, device=qfv.device)
-    # runs of several tokens take the wide form (a workgroup per 16 state columns; o through an fp32 scratch, then the norm)
-    scratch = torch.empty(n, heads * dv, dtype=torch.float32, device=qfv.device) if step.longest_run > 2 and dk <= 256 else None
+    # the wide form (a workgroup per 16 state columns; o through an fp32 scratch, then the norm) needs a scratch; the library
+    # picks the form (runs of several tokens, or batches too small to fill the chip with a workgroup per (sequence, head))
+    scratch = torch.empty(n, heads * dv, dtype=torch.float32, device=qfv.device) if dk <= 256 else None
     es = qfv.element_size()
     base = qfv.data_ptr()
     L.check(L.lib().ll_gated_linear_scan(
