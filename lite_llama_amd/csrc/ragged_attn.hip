@@ -10,6 +10,8 @@
 // The sink is a virtual key with score sink_h (not scaled) and a zero value: the running softmax simply STARTS at
 // (max = sink, sum = 1, output = 0).  A token's result depends only on its own position and on the cache rows of its
 // sequence, visited in a fixed order: how a prompt was cut into steps, or what else rides in the step, cannot change it.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -62,6 +64,87 @@ __global__ __launch_bounds__(256) void qk_norm_cache_kernel(
     if (wt) r *= ldv<DT>(wt, c);
     if (is_q) stv<DT>(q_out, (t * heads + item) * dk + c, r * temp);
     else stv<DT>(k_cache, (row * kv_heads + (item - heads)) * dk + c, r);
+  }
+}
+
+// sum over the 16 lanes of a DPP row (every lane of the row active); the result is in every lane of the row
+__device__ __forceinline__ float row16_sum(float v) {
+  float t;
+  t = ll_dpp_f32<0xB1>(v); v += t;   // quad_perm [1,0,3,2]
+  t = ll_dpp_f32<0x4E>(v); v += t;   // quad_perm [2,3,0,1]
+  t = ll_dpp_f32<0x124>(v); v += t;  // row_ror:4
+  t = ll_dpp_f32<0x128>(v); v += t;  // row_ror:8
+  return v;
+}
+
+// 16-byte form of the kernel above: one 16-lane row per (token, item), lane r of the row owns the 16-byte pieces r, r + 16, ..
+// of the head (up to four: widths <= 512 sixteen-bit / 256 fp32 channels, multiples of 8 / 4).
+template <int DT>
+__global__ __launch_bounds__(256) void qk_norm_cache_vec_kernel(
+    const void* __restrict__ qkv, int64_t ld, const void* __restrict__ q_w, const void* __restrict__ k_w, float eps,
+    float temp_coef, int temp_every, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ select,
+    void* __restrict__ q_out, void* __restrict__ k_cache, void* __restrict__ v_cache, int64_t n, int heads, int kv_heads, int dk,
+    int dv) {
+  constexpr int EPC = DT == LL_F32 ? 4 : 8;  // elements per 16-byte piece
+  typedef typename std::conditional<DT == LL_F32, float, uint16_t>::type elem;
+  const int items = heads + 2 * kv_heads;
+  const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+  if (row >= n * items) return;
+  const int r = threadIdx.x & 15;
+  const int64_t t = row / items;
+  const int item = (int)(row - t * items);
+  const bool is_q = item < heads, is_v = item >= heads + kv_heads;
+  const int width = is_v ? dv : dk;
+  const int64_t src = t * ld + (is_v ? (int64_t)(heads + kv_heads) * dk + (int64_t)(item - heads - kv_heads) * dv : (int64_t)item * dk);
+  const int pieces = width / EPC;
+  float val[4][EPC];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = r + 16 * j;
+    if (c < pieces) {
+      struct alignas(16) Piece { elem e[EPC]; };
+      const Piece pc = *reinterpret_cast<const Piece*>((const elem*)qkv + src + c * EPC);
+#pragma unroll
+      for (int e = 0; e < EPC; ++e) {
+        if constexpr (DT == LL_F32) val[j][e] = pc.e[e];
+        else val[j][e] = to_f32<DT>(pc.e[e]);
+        ss += val[j][e] * val[j][e];
+      }
+    }
+  }
+  float mul = 1.0f;
+  const void* wt = nullptr;
+  if (!is_v) {
+    ss = row16_sum(ss);
+    mul = 1.0f / sqrtf(ss / (float)dk + eps);
+    wt = is_q ? q_w : k_w;
+  }
+  float temp = 1.0f;
+  if (is_q && temp_coef != 0.f) temp = 1.0f + temp_coef * logf((float)((tok_pos[t] + 1) / temp_every) + 1.0f);
+  const int64_t crow = select[t];
+  elem* dst = is_q ? (elem*)q_out + (t * heads + item) * dk
+                   : is_v ? (elem*)v_cache + (crow * kv_heads + (item - heads - kv_heads)) * dv
+                          : (elem*)k_cache + (crow * kv_heads + (item - heads)) * dk;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = r + 16 * j;
+    if (c < pieces) {
+      struct alignas(16) Piece { elem e[EPC]; };
+      Piece o;
+#pragma unroll
+      for (int e = 0; e < EPC; ++e) {
+        float x = val[j][e];
+        if (!is_v) {
+          x *= mul;
+          if (wt) x *= ldv<DT>(wt, c * EPC + e);
+          if (is_q) x *= temp;
+        }
+        if constexpr (DT == LL_F32) o.e[e] = x;
+        else o.e[e] = from_f32<DT>(x);
+      }
+      *reinterpret_cast<Piece*>(dst + c * EPC) = o;
+    }
   }
 }
 
@@ -183,13 +266,18 @@ extern "C" int ll_qk_norm_cache(const void* qkv, int64_t ld, const void* q_w, co
   if (n == 0) return LL_OK;
   if (!qkv || !tok_pos || !select || !q_out || !k_cache || !v_cache) return LL_ERR_ARG;
   const int64_t waves = n * (heads + 2 * kv_heads);
-  const dim3 grid((unsigned)((waves + 3) / 4));
-#define CALL(DT)                                                                                                              \
-  qk_norm_cache_kernel<DT><<<grid, 256, 0, (hipStream_t)stream>>>(qkv, ld, q_w, k_w, eps, temp_coef, (int)temp_every, tok_pos, \
-                                                                 select, q_out, k_cache, v_cache, n, (int)heads, (int)kv_heads, \
-                                                                 (int)dk, (int)dv)
+  const int epc = dtype == LL_F32 ? 4 : 8;
+  const bool vec = dk % epc == 0 && dv % epc == 0 && ld % epc == 0 && dk <= 64 * epc && dv <= 64 * epc && ll_aligned16(qkv) &&
+                   ll_aligned16(q_out) && ll_aligned16(k_cache) && ll_aligned16(v_cache);
+  const dim3 grid((unsigned)((waves + 3) / 4)), grid_v((unsigned)((waves + 15) / 16));
+#define LL_QK_ARGS \
+  qkv, ld, q_w, k_w, eps, temp_coef, (int)temp_every, tok_pos, select, q_out, k_cache, v_cache, n, (int)heads, (int)kv_heads, (int)dk, (int)dv
+#define CALL(DT)                                                                                  \
+  if (vec) qk_norm_cache_vec_kernel<DT><<<grid_v, 256, 0, (hipStream_t)stream>>>(LL_QK_ARGS);     \
+  else qk_norm_cache_kernel<DT><<<grid, 256, 0, (hipStream_t)stream>>>(LL_QK_ARGS)
   LL_BY_DTYPE(dtype, CALL);
 #undef CALL
+#undef LL_QK_ARGS
   return LL_LAUNCH_CHECK();
 }
 
