@@ -496,7 +496,7 @@ __global__ __launch_bounds__(256) void head_rmsnorm_kernel(void* __restrict__ ou
 
 inline unsigned flat_grid(int64_t total) {
   const int64_t g = (total + 255) / 256;
-  return (unsigned)(g < 1 ? 1 : (g > 16384 ? 16384 : g));
+  return (unsigned)(g < 1 ? 1 : (g > (1 << 20) ? (1 << 20) : g));  // (one piece per thread up to 2^28 pieces: no ragged second pass)
 }
 
 }  // namespace

@@ -54,7 +54,7 @@ TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2}
 # mechanisms alone
 # ------------------------------------------------------------------------------------------------------------------- #
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("width", [72, 600])
+@pytest.mark.parametrize("width", [72, 70, 600])   # (70: not a multiple of 4 -> the plain, strided form)
 def test_add_norm_shift_reads_previous_rows_state_slots_and_zeros(dtype, width):
     from lite_llama_amd.kernels.norm_act import add_rmsnorm_shift
     from oracle import layered as O
