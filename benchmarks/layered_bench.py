@@ -159,22 +159,28 @@ def model_points(dev, dtype, width, heads, kv_heads, hd, ff, vocab, layers, pref
     res["layered_prefill"] = {"batch": b, "prompt": length, "ms": round(dt * 1e3, 2), "tokens_per_s": round(b * length / dt)}
     del runner
     b, ctx = decode
-    runner = RaggedRunner(model, b * (ctx + 64), b, 64, dev)
-    slots = [runner.admit() for _ in range(b)]
-    for lo in range(0, ctx, 256):
-        runner.step([(s, torch.randint(0, vocab, (min(256, ctx - lo),), generator=g).tolist()) for s in slots], [])
-    toks = [[1]] * b
-    for _ in range(3):
-        runner.step(list(zip(slots, toks)))
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        runner.step(list(zip(slots, toks)))
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / steps
-    res["layered_decode"] = {"batch": b, "ctx": ctx, "ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(b / dt),
-                             "launches": "eager (host builds the step's vectors every step)"}
-    del runner, model
+    for captured in (False, True):
+        runner = RaggedRunner(model, b * (ctx + 64), b, 64, dev, capture_decode=captured)
+        slots = [runner.admit() for _ in range(b)]
+        for lo in range(0, ctx, 256):
+            runner.step([(s, torch.randint(0, vocab, (min(256, ctx - lo),), generator=g).tolist()) for s in slots], [])
+        toks = [[1]] * b
+        for _ in range(3):
+            runner.step(list(zip(slots, toks)))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            runner.step(list(zip(slots, toks)))
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        res["layered_decode_captured" if captured else "layered_decode"] = {
+            "batch": b, "ctx": ctx, "ms_per_step": round(dt * 1e3, 3), "tokens_per_s": round(b / dt),
+            "launches": ("one hipGraph per step (one small host-to-device copy of the step's vectors in front)" if captured
+                         else "eager (host builds the step's vectors every step)")}
+        if captured:
+            res["layered_decode_captured"]["replays"] = runner.replays
+        del runner
+    del model
     torch.cuda.empty_cache()
     # the closest llama-shaped model: same widths, rotary attention + swiglu MLP in every layer
     cgeo = ModelGeometry("bench", width, layers, heads, kv_heads, hd, ff, vocab)

@@ -43,7 +43,7 @@ def _generate(args) -> int:
         page = args.page_size
         pool = args.max_tokens or sum(-(-(len(p) + args.max_new_tokens) // page) * page for p in prompts[:args.max_requests])
         engine = GenerationEngine(model, pool, max_requests=args.max_requests, block_size=page,
-                                  max_step_tokens=args.max_step_tokens, seed=args.seed)
+                                  max_step_tokens=args.max_step_tokens, seed=args.seed, capture_decode=args.capture_decode)
         outs = engine.generate(prompts, params)
     else:
         import types
@@ -88,6 +88,7 @@ def main(argv=None) -> int:
     g.add_argument("--max-step-tokens", type=int, default=512)
     g.add_argument("--page-size", type=int, default=64)
     g.add_argument("--seed", type=int, default=0)
+    g.add_argument("--capture-decode", action="store_true", help="layered models: replay decode-only steps from hipGraphs")
     sub.add_parser("trace", add_help=False)
     b = sub.add_parser("build")
     b.add_argument("--part", default=None)

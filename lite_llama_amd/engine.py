@@ -49,10 +49,12 @@ class _Span:
 
 class GenerationEngine:
     def __init__(self, model, max_tokens: int, max_requests: int = 4, block_size: int = 64, max_step_tokens: int = 512,
-                 device="cuda", seed: int = 0):
+                 device="cuda", seed: int = 0, capture_decode: bool = False):
         """``max_tokens``: size of the cache pool (tokens over all live requests, block-rounded per request);
-        ``max_step_tokens``: the most tokens one step carries -- decode tokens first, the rest goes to prompt portions."""
-        self.runner = RaggedRunner(model, max_tokens, max_requests, block_size, device)
+        ``max_step_tokens``: the most tokens one step carries -- decode tokens first, the rest goes to prompt portions;
+        ``capture_decode``: steps that carry decode tokens only are replayed from a hipGraph per (running set, context
+        partitions) cell (``RaggedRunner._decode_step_captured``)."""
+        self.runner = RaggedRunner(model, max_tokens, max_requests, block_size, device, capture_decode=capture_decode)
         self.max_step_tokens = max(1, int(max_step_tokens))
         self.device = torch.device(device)
         self._waiting: deque[_Request] = deque()

@@ -42,13 +42,22 @@ class RaggedStep:
         return self.seq_slot
 
 
+class _DecodeCell:
+    """A captured decode step: the graph, the persistent packed step vectors it reads, the logits it leaves."""
+
+    graph = None
+    packed = None
+    rows = None
+    logits = None
+
+
 class RaggedRunner:
     """Model + cache + request slots.  ``admit()`` hands out a slot, ``step()`` runs one ragged step and returns the logits of
     the asked rows, ``release()`` gives a request's blocks and slot back.  Nothing is kept per request on the host but its
     length and parity; blocks are popped and pushed on the device (``PagedStateCache``)."""
 
     def __init__(self, model, max_tokens: int, max_requests: int = 4, block_size: int = 64, device="cuda",
-                 max_seq_len: int | None = None):
+                 max_seq_len: int | None = None, capture_decode: bool = False):
         """``max_tokens``: the most tokens that live requests hold at any time, each request's count rounded up to a multiple
         of ``block_size``: the block pool is made for that many (plus the junk block), not for ``max_requests`` full-length
         sequences."""
@@ -66,6 +75,11 @@ class RaggedRunner:
         self._free_slots = list(range(max_requests))
         self._len: dict[int, int] = {}
         self._parity: dict[int, int] = {}
+        # captured decode steps (opt-in): one hipGraph per (slots riding, context partitions) cell, see _decode_cell
+        self.capture_decode = bool(capture_decode)
+        self._cells: dict[tuple, "_DecodeCell"] = {}
+        self._sightings: dict[tuple, int] = {}
+        self.replays = 0
 
     # ------------------------------------------------------------------ requests ---- #
     @property
@@ -99,9 +113,9 @@ class RaggedRunner:
             self._free_slots.append(s)
 
     # ------------------------------------------------------------------ one step ---- #
-    def build_step(self, entries: Sequence[tuple[int, Sequence[int]]]) -> tuple[RaggedStep, torch.Tensor]:
-        """``entries``: ``(slot, next tokens)`` per sequence, every slot at most once.  Reserves blocks for the new tokens and
-        advances the host-side lengths and parities."""
+    def _plan(self, entries: Sequence[tuple[int, Sequence[int]]]):
+        """``entries``: ``(slot, next tokens)`` per sequence, every slot at most once.  Checks the step against the pool, builds
+        its vectors as host lists and advances the host-side lengths and parities."""
         if not entries:
             raise ValueError("an empty step")
         slots = [s for s, _ in entries]
@@ -125,22 +139,34 @@ class RaggedRunner:
             tok_pos += range(f, f + c)
             pick += range(i * longest + longest - c, (i + 1) * longest)
             tokens += [int(t) for t in toks]
-        # every vector of the step crosses to the device in ONE copy: a packed int32 tensor, sliced into views
         parts = [tok_seq, tok_pos, starts, first, slots, [self._parity[s] for s in slots], new_len, pick, tokens]
-        packed = torch.tensor([v for part in parts for v in part], dtype=torch.int32).to(self.device, non_blocking=True)
-        views, at = [], 0
-        for part in parts:
-            views.append(packed[at:at + len(part)])
-            at += len(part)
-        v_tok_seq, v_tok_pos, v_starts, v_first, v_slots, v_parity, v_new_len, v_pick, v_tokens = views
-        rows = self.cache.extend(v_slots, v_new_len, longest, self.token_table)
-        select = rows.reshape(-1)[v_pick].contiguous()
-        step = RaggedStep(num_tokens=len(tokens), num_seqs=len(entries), tok_seq=v_tok_seq, tok_pos=v_tok_pos, select=select,
-                          seq_start=v_starts, seq_first_pos=v_first, seq_slot=v_slots, seq_parity=v_parity, longest_run=longest,
-                          longest_context=max(new_len))
         for s, n in zip(slots, new_len):
             self._len[s] = n
             self._parity[s] ^= 1
+        return parts, longest, max(new_len)
+
+    @staticmethod
+    def _views(packed: torch.Tensor, sizes):
+        views, at = [], 0
+        for n in sizes:
+            views.append(packed[at:at + n])
+            at += n
+        return views
+
+    def build_step(self, entries: Sequence[tuple[int, Sequence[int]]]) -> tuple[RaggedStep, torch.Tensor]:
+        """The step's device vectors: every one of them crosses to the device in ONE copy (a packed int32 tensor, sliced into
+        views); blocks for the new tokens are reserved on the device."""
+        parts, longest, longest_context = self._plan(entries)
+        packed = torch.tensor([v for part in parts for v in part], dtype=torch.int32).to(self.device, non_blocking=True)
+        return self._step_from(packed, [len(p) for p in parts], len(entries), longest, longest_context)
+
+    def _step_from(self, packed, sizes, num_seqs, longest, longest_context):
+        v_tok_seq, v_tok_pos, v_starts, v_first, v_slots, v_parity, v_new_len, v_pick, v_tokens = self._views(packed, sizes)
+        rows = self.cache.extend(v_slots, v_new_len, longest, self.token_table)
+        select = rows.reshape(-1)[v_pick].contiguous() if longest > 1 else rows.reshape(-1)
+        step = RaggedStep(num_tokens=v_tokens.numel(), num_seqs=num_seqs, tok_seq=v_tok_seq, tok_pos=v_tok_pos, select=select,
+                          seq_start=v_starts, seq_first_pos=v_first, seq_slot=v_slots, seq_parity=v_parity, longest_run=longest,
+                          longest_context=longest_context)
         return step, v_tokens
 
     @torch.no_grad()
@@ -149,15 +175,59 @@ class RaggedRunner:
         """Run the entries as ONE batch.  ``logits_rows``: flat token indices (in entry order) whose logits are wanted; ``None``
         = the last token of every entry; an empty list = none (the step still fills cache and state).  Returns
         ``[rows, vocab]`` logits in the model's dtype, or ``None``."""
-        step, token_ids = self.build_step(entries)
         if logits_rows is None:
             logits_rows, at = [], 0
             for _, toks in entries:
                 at += len(toks)
                 logits_rows.append(at - 1)
-        rows = torch.tensor(list(logits_rows), dtype=torch.long, device=self.device) if len(logits_rows) else None
-        out = self.model(token_ids, step, self.cache, self.token_table, logits_rows=rows, collect_layers=collect_layers)
-        return out
+        logits_rows = list(logits_rows)
+        if (self.capture_decode and collect_layers is None and all(len(t) == 1 for _, t in entries)
+                and logits_rows == list(range(len(entries)))):
+            return self._decode_step_captured(entries)
+        step, token_ids = self.build_step(entries)
+        rows = torch.tensor(logits_rows, dtype=torch.long, device=self.device) if logits_rows else None
+        return self.model(token_ids, step, self.cache, self.token_table, logits_rows=rows, collect_layers=collect_layers)
+
+    # ------------------------------------------------------------------ captured decode steps ---- #
+    def _decode_step_captured(self, entries):
+        """A step in which every sequence brings its one decoded token and every row's logits are wanted.  Such steps repeat
+        with the same slots for as long as nobody finishes: the SECOND time a (slots, context partitions) cell is seen its
+        launch list is captured as one hipGraph over persistent step vectors, and from then on a step is one small host-to-
+        device copy plus one graph launch.  The first sighting runs eagerly (which also sizes every workspace the capture
+        needs).  The returned logits live in the graph's memory: use them before the next step of the same cell."""
+        from .. import _lib as L
+
+        part = int(L.lib().ll_ragged_attention_partition()) if L.has("ll_ragged_attention_partition") else 256
+        parts, longest, longest_context = self._plan(entries)
+        key = (tuple(s for s, _ in entries), -(-longest_context // part))
+        host = torch.tensor([v for p in parts for v in p], dtype=torch.int32)
+        cell = self._cells.get(key)
+        if cell is None:
+            self._sightings[key] = self._sightings.get(key, 0) + 1
+            if self._sightings[key] < 2:
+                step, token_ids = self._step_from(host.to(self.device), [len(p) for p in parts], len(entries), 1, longest_context)
+                rows = torch.arange(len(entries), device=self.device)
+                return self.model(token_ids, step, self.cache, self.token_table, logits_rows=rows)
+            cell = self._capture_cell(key, host, [len(p) for p in parts], len(entries), key[1] * part)
+        cell.packed.copy_(host)   # (pageable source: the copy has left the host buffer when this returns)
+        cell.graph.replay()
+        self.replays += 1
+        return cell.logits
+
+    def _capture_cell(self, key, host, sizes, num_seqs, context_bound):
+        while len(self._cells) >= 8:                      # a handful of cells at a time: the oldest goes
+            self._cells.pop(next(iter(self._cells)))
+        cell = _DecodeCell()
+        cell.packed = host.to(self.device)
+        cell.rows = torch.arange(num_seqs, device=self.device)
+        torch.cuda.synchronize()
+        cell.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(cell.graph):
+            step, token_ids = self._step_from(cell.packed, sizes, num_seqs, 1, context_bound)
+            cell.logits = self.model(token_ids, step, self.cache, self.token_table, logits_rows=cell.rows)
+        self._cells[key] = cell
+        self._sightings.pop(key, None)
+        return cell
 
     def check_errors(self) -> None:
         """Synchronising read of the block pool's sticky error word."""

@@ -112,7 +112,7 @@ class _FakeRunner:
 def _engine(monkeypatch, max_tokens, max_requests, block, budget):
     from lite_llama_amd import engine as E
 
-    monkeypatch.setattr(E, "RaggedRunner", lambda model, mt, mr, bs, dev: _FakeRunner(mt, mr, bs))
+    monkeypatch.setattr(E, "RaggedRunner", lambda model, mt, mr, bs, dev, capture_decode=False: _FakeRunner(mt, mr, bs))
     eng = E.GenerationEngine(None, max_tokens, max_requests, block, budget, device="cpu")
     monkeypatch.setattr(eng, "_sample", lambda logits, reqs: [int(v) for v in logits.argmax(-1)])
     return eng, E

@@ -390,6 +390,35 @@ def test_bfloat16_model_tracks_the_oracle_and_its_own_portions(tmp_path_factory,
     assert (parts - whole).pow(2).mean().sqrt().item() < 0.03 * spread      # same rounding points, other GEMM shapes
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_captured_decode_steps_replay_like_eager_ones(tmp_path_factory, dtype):
+    """Decode-only steps from a hipGraph per (running set, context partitions) cell against the same steps launched eagerly:
+    many replays with eager work between them (a neighbour's prompt portions change the running set and come back), a context
+    that grows across a partition edge (a second cell for the same slots), every replay compared."""
+    from lite_llama_amd.executor.ragged import RaggedRunner
+
+    model, cfg, _, _ = _model(tmp_path_factory, "loop0", dtype)
+    a, b = T.prompt(cfg, 290, seed=21), T.prompt(cfg, 40, seed=22)
+    eager = RaggedRunner(model, 512, 2, block_size=16, device=DEV)
+    graph = RaggedRunner(model, 512, 2, block_size=16, device=DEV, capture_decode=True)
+    out = {"eager": [], "graph": []}
+    for name, r in (("eager", eager), ("graph", graph)):
+        sa, sb = r.admit(), r.admit()
+        r.step([(sa, a[:240])], [])
+        for i in range(240, 262):                                   # one sequence decoding: 256 is a partition edge
+            out[name].append(r.step([(sa, a[i:i + 1])]).float().cpu().clone())
+        r.step([(sa, a[262:263]), (sb, b[:30])], [])                 # a mixed step in between (eager in both runners)
+        for i in range(10):                                         # two sequences decoding together
+            out[name].append(r.step([(sa, a[263 + i:264 + i]), (sb, b[30 + i:31 + i])]).float().cpu().clone())
+        r.release([sb])
+        for i in range(273, 290):                                   # back to the first running set: its cell is replayed again
+            out[name].append(r.step([(sa, a[i:i + 1])]).float().cpu().clone())
+        r.check_errors()
+    assert graph.replays >= 40 and eager.replays == 0
+    for e, g2 in zip(out["eager"], out["graph"]):
+        assert torch.allclose(e, g2, rtol=0, atol=1e-6 if dtype == torch.float32 else 2e-2), (e - g2).abs().max()
+
+
 # ------------------------------------------------------------------------------------------------------------------- #
 # entry points: engine, command line, trace replay
 # ------------------------------------------------------------------------------------------------------------------- #
@@ -403,6 +432,8 @@ def test_engine_generates_greedily_like_the_oracle(tmp_path_factory):
     outs = engine.generate(prompts, SamplingParams(max_new_tokens=6))
     for p, o in zip(prompts, outs):
         assert o == O.greedy(cfg, tens, p, 6)
+    captured = GenerationEngine(model, max_tokens=96, max_requests=3, block_size=8, max_step_tokens=10, device=DEV, capture_decode=True)
+    assert captured.generate(prompts, SamplingParams(max_new_tokens=6)) == outs and captured.runner.replays > 0
     assert engine.runner.cache.free_blocks == engine.runner.total_blocks and engine.runner.free_slots == 3
     sampled = engine.generate(prompts[:2], SamplingParams(max_new_tokens=5, temperature=0.8, top_p=0.9, repetition_penalty=1.2))
     assert [len(s) for s in sampled] == [5, 5] and all(0 <= t < cfg["vocab"] for s in sampled for t in s)
