@@ -370,8 +370,8 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(
           if (r < rows) {
             const int k = g + r * kg;
             const float fg = sf[tt * dk + k];
-            S[r] = fg * S[r] + (1.0f - fg) * val;
-            acc += S[r] * sq[tt * dk + k];
+            S[r] = __builtin_fmaf(fg, S[r], (1.0f - fg) * val);
+            acc = __builtin_fmaf(S[r], sq[tt * dk + k], acc);
           }
         }
         sp[(tt * kg + g) * dv + c] = acc;
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(
 // costs per token.  Thread (kg, c): column c of the slice, rows kg, kg + 16, ...  The per-head output norm needs all dv
 // columns: o goes to an fp32 scratch [n, heads dv] and head_rmsnorm_kernel finishes.  The state update is the expression of
 // the form above, so both leave the same state bits.
-template <int DT, int RMAX>
+template <int DT, int RMAX, bool EXACT>   // EXACT: dk == 16 RMAX, every thread owns RMAX rows (no per-row guards)
 __global__ __launch_bounds__(256) void gated_linear_scan_wide_kernel(
     const void* __restrict__ q, const void* __restrict__ f, const void* __restrict__ v, int64_t ld, const void* __restrict__ f_bias,
     const void* __restrict__ lower, float* __restrict__ o_scratch, int heads, int dk, int dv, int tb,
@@ -423,11 +423,9 @@ __global__ __launch_bounds__(256) void gated_linear_scan_wide_kernel(
   const int tid = threadIdx.x, col = tid & 15, kg = tid >> 4;
   const bool active = c0 + col < dv && kg < dk;
   const int rows = kg < dk ? (dk - kg + 15) / 16 : 0;
-  float* sf = lds;                 // [tb][dk] forget gates
-  float* su = sf + tb * dk;        // [tb][dk] 1 - gate
-  float* sq = su + tb * dk;        // [tb][dk] queries
-  float* sv = sq + tb * dk;        // [tb][16] values of the slice
-  float* sp = sv + tb * 16;        // [tb][16 groups][16] partial outputs
+  f32x4* sg = reinterpret_cast<f32x4*>(lds);          // [tb][dk] (gate, 1 - gate, query, -): one 16-byte read per state row
+  float* sv = lds + 4 * tb * dk;                       // [tb][16] values of the slice
+  float* sp = sv + tb * 16;                            // [tb][16 groups][16] partial outputs
   const int t0 = seq_start[b], t1 = seq_start[b + 1];
   float* st = state + ((int64_t)seq_slot[b] * heads + head) * dk * dv + c0 + col;
   const bool carry = seq_first_pos[b] > 0;
@@ -442,10 +440,8 @@ __global__ __launch_bounds__(256) void gated_linear_scan_wide_kernel(
       const int64_t at = (int64_t)(base + tt) * ld + head * dk + k;
       const float lo = ldv<DT>(lower, head * dk + k);
       const float fg = lo + (1.0f - lo) * gate_sigmoid<DT>(ldv<DT>(f, at) + ldv<DT>(f_bias, head * dk + k));
-      sf[i] = fg;
-      su[i] = 1.0f - fg;
       const float qv = ldv<DT>(q, at);
-      sq[i] = qv * gate_sigmoid<DT>(qv);
+      sg[i] = f32x4{fg, 1.0f - fg, qv * gate_sigmoid<DT>(qv), 0.f};
     }
     for (int i = tid; i < nt * 16; i += 256) {
       const int tt = i >> 4, cc = i & 15;
@@ -457,10 +453,10 @@ __global__ __launch_bounds__(256) void gated_linear_scan_wide_kernel(
       float acc = 0.f;
 #pragma unroll
       for (int r = 0; r < RMAX; ++r) {
-        if (r < rows) {
-          const int k = tt * dk + kg + 16 * r;
-          S[r] = sf[k] * S[r] + su[k] * val;
-          acc += S[r] * sq[k];
+        if (EXACT || r < rows) {
+          const f32x4 gq = sg[tt * dk + kg + 16 * r];
+          S[r] = __builtin_fmaf(gq[0], S[r], gq[1] * val);   // (the expression of the fused form: both leave the same bits)
+          acc = __builtin_fmaf(S[r], gq[2], acc);
         }
       }
       sp[(tt * 16 + kg) * 16 + col] = acc;
@@ -593,16 +589,19 @@ extern "C" int ll_gated_linear_scan(const void* q, const void* f, const void* v,
     // wide form + output norm: runs of several tokens (prompt portions, mixed steps), and decode batches too small to fill the
     // chip with one workgroup per (sequence, head)
     const int tb = dk <= 128 ? 16 : 8;
-    const size_t lds = sizeof(float) * (size_t)(tb * (3 * dk + 16 + 256));
+    const size_t lds = sizeof(float) * (size_t)(tb * (4 * dk + 16 + 256));
     const dim3 grid((unsigned)batch, (unsigned)heads, (unsigned)((dv + 15) / 16));
     const int rmax = (int)((dk + 15) / 16);
-#define CALL_W(DT, R)                                                                                                          \
-  gated_linear_scan_wide_kernel<DT, R><<<grid, 256, lds, st>>>(q, f, v, ld, f_bias, lower, scratch, (int)heads, (int)dk, (int)dv, \
-                                                               tb, seq_start, seq_first_pos, seq_slot, state)
-#define CALL(DT)                     \
-  if (rmax <= 4) CALL_W(DT, 4);      \
-  else if (rmax <= 8) CALL_W(DT, 8); \
-  else CALL_W(DT, 16)
+#define CALL_W(DT, R, E)                                                                                                       \
+  gated_linear_scan_wide_kernel<DT, R, E><<<grid, 256, lds, st>>>(q, f, v, ld, f_bias, lower, scratch, (int)heads, (int)dk,    \
+                                                                  (int)dv, tb, seq_start, seq_first_pos, seq_slot, state)
+#define CALL(DT)                                \
+  if (dk == 64) CALL_W(DT, 4, true);            \
+  else if (dk == 128) CALL_W(DT, 8, true);      \
+  else if (dk == 256) CALL_W(DT, 16, true);     \
+  else if (rmax <= 4) CALL_W(DT, 4, false);     \
+  else if (rmax <= 8) CALL_W(DT, 8, false);     \
+  else CALL_W(DT, 16, false)
     LL_BY_DTYPE(dtype, CALL);
 #undef CALL
 #undef CALL_W
