@@ -593,11 +593,13 @@ int ll_qk_norm_cache(const void* qkv, int64_t ld, const void* q_w, const void* k
                      void* v_cache, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int dtype,
                      void* stream);
 /* Causal softmax attention of every token against positions 0 .. tok_pos[t] of its sequence (cache rows through
- * token_table[seq_req[tok_seq[t]]][pos]); score = (q . k) scale; sink [heads] or NULL adds exp(sink_h) to the denominator. */
+ * token_table[seq_req[tok_seq[t]]][pos]); score = (q . k) scale; sink [heads] or NULL adds exp(sink_h) to the denominator.
+ * window > 0: only the last `window` positions (the token's own included) are seen.  k_stride / v_stride: elements between
+ * cache rows (>= kv_heads dk / kv_heads dv; the value rows may be a column range of the key rows). */
 int ll_ragged_attention(const void* q, const void* k_cache, const void* v_cache, const int32_t* token_table,
                         int64_t tt_stride, const int32_t* seq_req, const int32_t* tok_seq, const int32_t* tok_pos,
                         const void* sink, float scale, void* out, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk,
-                        int64_t dv, int dtype, void* stream);
+                        int64_t dv, int64_t k_stride, int64_t v_stride, int64_t window, int dtype, void* stream);
 /* MFMA form for 16-bit storage dtypes (dk, dv multiples of 8, <= 256).  decode == 0: prompt portions (16 consecutive tokens
  * of a run per wave; longest_run = most tokens a sequence brings).  decode != 0: every sequence brings one token (n == batch);
  * the query heads of a key/value head share a wave, the context is cut into partitions of ll_ragged_attention_partition()
@@ -609,7 +611,64 @@ int ll_ragged_attention_mfma(const void* q, const void* k_cache, const void* v_c
                              int64_t tt_stride, const int32_t* seq_req, const int32_t* seq_start,
                              const int32_t* seq_first_pos, const void* sink, float scale, void* out, int64_t n,
                              int64_t batch, int64_t longest_run, int64_t longest_context, int decode, float* partials,
-                             int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int dtype, void* stream);
+                             int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int64_t k_stride, int64_t v_stride,
+                             int64_t window, int dtype, void* stream);
+
+/* ---- sublayers between two grouped norms with a gated residual branch (csrc/group_norm.hip) --------------------------------
+ * ll_gated_group_norm: with y: s = (sum of `parts` rows y[t][p][:] + shared_scale[t] * shared[t][:]) * sigmoid(gate[t][:] +
+ * gate_bias) (shared, gate, gate_bias may be NULL; gate rows have stride gate_ld), x_out = x_in + groupnorm(s) * post_w, and,
+ * when h_out is given, h_out = groupnorm(x_out) * next_w.  Without y: h_out = groupnorm(x_in) * next_w.  groupnorm: the row in
+ * `groups` equal consecutive parts, each divided by sqrt(mean(part^2) + eps).  x_out may be x_in. */
+int ll_gated_group_norm(const float* x_in, float* x_out, void* h_out, const void* y, int64_t parts, const void* shared,
+                        const float* shared_scale, const void* gate, int64_t gate_ld, const void* gate_bias,
+                        const void* post_w, const void* next_w, int64_t n, int64_t width, int64_t groups, float eps,
+                        int dtype, void* stream);
+/* out [n, ff] = act(gate[t][j]) * up[t][j], gate / up rows of stride gate_ld / up_ld; kind 0: silu, 1: gelu (tanh form),
+ * 2: sigmoid. */
+int ll_glu_act(void* out, const void* gate, int64_t gate_ld, const void* up, int64_t up_ld, int64_t n, int64_t ff, int kind,
+               int dtype, void* stream);
+/* x <- cap * tanh(x / cap), in place. */
+int ll_softcap(void* x, int64_t n, float cap, int dtype, void* stream);
+/* minGRU: rows [z | x | g] (three pointers, one stride ld): z = sigmoid(z_raw + z_bias), u = x_raw + x_bias, candidate u + 1/2
+ * (u >= 0) or sigmoid(u); S <- (1 - z) S + z candidate per channel, out = S * silu(g_raw).  state [slots][width] fp32 (read when
+ * seq_first_pos > 0, written at the end of the run). */
+int ll_mingru_scan(const void* z, const void* x, const void* g, int64_t ld, const void* z_bias, const void* x_bias,
+                   void* out, int64_t batch, int64_t width, const int32_t* seq_start, const int32_t* seq_first_pos,
+                   const int32_t* seq_slot, float* state, int dtype, void* stream);
+
+/* ---- attention over a shared latent (csrc/latent_attn.hip) ------------------------------------------------------------------
+ * ll_latent_kv_prep: rows (stride ld) hold the latent [rank] and the rotated key part [rot] at column kv_off: the cache row
+ * select[t] (stride cache_stride) receives [latent RMS-normed * kv_norm_w | key part rotated at tok_pos[t]]; with q_rank > 0
+ * the columns q_off .. q_off + q_rank are RMS-normed with q_norm_w into q_out [n, q_rank].  Rotation: entry 2i with 2i + 1 by
+ * the angle tok_pos * freq[i] (i < pairs), cos and sin times amp; entries from 2 pairs on pass unchanged.
+ * ll_rotate_pairs: the same rotation of the `rot` entries at q_off of every head of q (token / head strides given), written to
+ * out[(t heads + h) out_head_stride + out_off ..]. */
+int ll_latent_kv_prep(const void* rows, int64_t ld, int64_t kv_off, int64_t rank, int64_t rot, const void* kv_norm_w,
+                      float eps, const float* freq, int64_t pairs, float amp, const int32_t* tok_pos,
+                      const int32_t* select, void* cache, int64_t cache_stride, int64_t q_off, int64_t q_rank,
+                      const void* q_norm_w, void* q_out, int64_t n, int dtype, void* stream);
+int ll_rotate_pairs(const void* q, int64_t q_tok_stride, int64_t q_head_stride, int64_t q_off, int64_t rot,
+                    const float* freq, int64_t pairs, float amp, const int32_t* tok_pos, void* out,
+                    int64_t out_head_stride, int64_t out_off, int64_t n, int64_t heads, int dtype, void* stream);
+
+/* ---- mixture of experts with a sigmoid router over expert groups (csrc/moe_sparse.hip) --------------------------------------
+ * ll_group_router: scores = sigmoid(W_router h) in fp32; experts in group_count equal groups of neighbours, group score = sum
+ * of its two best, the best group_keep groups stay eligible; ids [n, top] / weights [n, top] (fp32) = the top eligible experts
+ * by score and score / (sum + 1e-20) * route_scale.  w_extra [width] (or NULL): extra_scale[t] = sigmoid(w_extra . h).
+ * ll_moe_sort: slots sorted by expert in blocks of ll_moe_rows_block() rows (counts: int32 scratch [experts]; sorted
+ * [num_slots + experts (block - 1)], block_expert [ceil(that / block)], num_post [1]).
+ * ll_moe_rows_gemm: glu != 0: w [experts][2 N][K] (gate rows, then up rows), out[slot] = silu(a Wg^T) * (a Wu^T) with
+ * a = row slot / a_div; glu == 0: w [experts][N][K], out[slot] = (a W^T) * slot_weight[slot]. */
+int ll_group_router(const void* h, int64_t h_ld, const void* w_router, const void* w_extra, int64_t n, int64_t width,
+                    int64_t experts, int64_t top, int64_t group_count, int64_t group_keep, float route_scale,
+                    int32_t* ids, float* weights, float* extra_scale, int dtype, void* stream);
+int64_t ll_moe_rows_block(void);
+int ll_moe_sort(const int32_t* ids, int64_t num_slots, int64_t experts, int32_t* counts, int32_t* sorted,
+                int32_t* block_expert, int32_t* num_post, void* stream);
+int ll_moe_rows_gemm(const void* a, int64_t a_ld, int64_t a_div, const void* w, int64_t w_stride_e, int64_t K, int64_t N,
+                     int glu, const float* slot_weight, void* out, int64_t out_ld, const int32_t* sorted,
+                     const int32_t* block_expert, const int32_t* num_post, int64_t num_slots, int64_t experts, int dtype,
+                     void* stream);
 
 #ifdef __cplusplus
 }

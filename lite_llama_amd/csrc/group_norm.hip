@@ -1,0 +1,269 @@
+// Layers whose sublayers are wrapped in TWO norms and a learned gate on the residual branch (32-bit residual stream):
+//
+//     x <- x + norm_b( f(norm_a(x)) * sigmoid(W_r norm_a(x) + b_r) )
+//
+// with RMS norms taken over GROUPS: the row is cut into `groups` equal consecutive parts, each divided by its own root mean
+// square, then the whole is multiplied by the weight.
+//
+//   ll_gated_group_norm   closes one sublayer and opens the next in ONE launch: the sublayer's result (one row per token, or the
+//                         sum of several rows -- the experts a token chose -- plus a scaled shared row) times the sigmoid of its
+//                         gate logits, grouped norm with the post weight, residual add in fp32, then the grouped norm that feeds
+//                         the next sublayer (or the output head).  Without a pending result it is the plain grouped norm.
+//   ll_glu_act            act(gate) * up, gate and up two row-strided column ranges (act: silu, the tanh form of gelu, sigmoid)
+//
+// Storage dtype DT = LL_F16 / LL_BF16 / LL_F32 for activations and weights; sums, norms, gates and the residual are fp32.
+#include "common.h"
+
+namespace {
+
+template <int DT>
+__device__ __forceinline__ float ldv(const void* p, int64_t i) {
+  if constexpr (DT == LL_F32) return ((const float*)p)[i];
+  else return to_f32<DT>(((const uint16_t*)p)[i]);
+}
+template <int DT>
+__device__ __forceinline__ void stv(void* p, int64_t i, float v) {
+  if constexpr (DT == LL_F32) ((float*)p)[i] = v;
+  else ((uint16_t*)p)[i] = from_f32<DT>(v);
+}
+
+// sum over a 256-thread workgroup in a fixed order (wave sums, then the four waves in order)
+__device__ __forceinline__ float block_sum256(float v, float* lds4) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds4[wave] = v;
+  __syncthreads();
+  return ((lds4[0] + lds4[1]) + lds4[2]) + lds4[3];
+}
+
+template <bool EXACT>
+__device__ __forceinline__ float sigmoid_f(float v) {
+  if constexpr (EXACT) return 1.0f / (1.0f + expf(-v));
+  else return ll_sigmoidf(v);
+}
+
+// One workgroup per token; thread i owns elements i, i + 256, ... of every group (the same elements in every pass, so a
+// thread re-reads only what it wrote itself).  NV > 0: the gated value of a thread's elements stays in registers between the
+// passes (rows of up to 256 NV elements per group pass); NV == 0: recomputed from memory.
+template <int DT>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(
+    const float* x_in, float* x_out, void* __restrict__ h_out, const void* __restrict__ y, int parts,
+    const void* __restrict__ shared, const float* __restrict__ shared_scale, const void* __restrict__ gate, int64_t gate_ld,
+    const void* __restrict__ gate_bias, const void* __restrict__ post_w, const void* __restrict__ next_w, int width, int groups,
+    float eps) {
+  constexpr bool EXACT = DT == LL_F32;
+  __shared__ float red[4];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int gs = width / groups;
+  const float* xr = x_in + t * width;
+  float* xo = x_out + t * width;
+  const float sscale = shared ? shared_scale[t] : 0.f;
+
+  auto branch = [&](int i) -> float {   // the sublayer's gated result at element i
+    float s = 0.f;
+    for (int p = 0; p < parts; ++p) s += ldv<DT>(y, (t * parts + p) * (int64_t)width + i);
+    if (shared) s += sscale * ldv<DT>(shared, t * (int64_t)width + i);
+    if (gate) {
+      float r = ldv<DT>(gate, t * gate_ld + i);
+      if (gate_bias) r += ldv<DT>(gate_bias, i);
+      s *= sigmoid_f<EXACT>(r);
+    }
+    return s;
+  };
+
+  for (int g = 0; g < groups; ++g) {
+    const int lo = g * gs, hi = lo + gs;
+    if (y) {
+      float ss = 0.f;
+      for (int i = lo + tid; i < hi; i += 256) {
+        const float s = branch(i);
+        ss += s * s;
+      }
+      ss = block_sum256(ss, red);
+      const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+      float s2 = 0.f;
+      for (int i = lo + tid; i < hi; i += 256) {
+        const float v = xr[i] + branch(i) * inv * ldv<DT>(post_w, i);
+        xo[i] = v;
+        s2 += v * v;
+      }
+      s2 = block_sum256(s2, red);
+      if (h_out) {
+        const float inv2 = 1.0f / sqrtf(s2 / (float)gs + eps);
+        for (int i = lo + tid; i < hi; i += 256) stv<DT>(h_out, t * (int64_t)width + i, xo[i] * inv2 * ldv<DT>(next_w, i));
+      }
+    } else {
+      float s2 = 0.f;
+      for (int i = lo + tid; i < hi; i += 256) {
+        const float v = xr[i];
+        s2 += v * v;
+      }
+      s2 = block_sum256(s2, red);
+      const float inv2 = 1.0f / sqrtf(s2 / (float)gs + eps);
+      for (int i = lo + tid; i < hi; i += 256) stv<DT>(h_out, t * (int64_t)width + i, xr[i] * inv2 * ldv<DT>(next_w, i));
+    }
+  }
+}
+
+// Register-cached form: a thread keeps the gated values of its elements (and then the new residual) between the passes, so
+// every input is read once.  Same arithmetic and reduction order as the plain form.  Needs width / groups <= 256 NV.
+template <int DT, int NV>
+__global__ __launch_bounds__(256) void gated_group_norm_cached_kernel(
+    const float* x_in, float* x_out, void* __restrict__ h_out, const void* __restrict__ y, int parts,
+    const void* __restrict__ shared, const float* __restrict__ shared_scale, const void* __restrict__ gate, int64_t gate_ld,
+    const void* __restrict__ gate_bias, const void* __restrict__ post_w, const void* __restrict__ next_w, int width, int groups,
+    float eps) {
+  constexpr bool EXACT = DT == LL_F32;
+  __shared__ float red[4];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int gs = width / groups;
+  const float* xr = x_in + t * width;
+  float* xo = x_out + t * width;
+  const float sscale = shared ? shared_scale[t] : 0.f;
+  for (int g = 0; g < groups; ++g) {
+    const int lo = g * gs, hi = lo + gs;
+    float val[NV];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int i = lo + tid + 256 * k;
+      float s = 0.f;
+      if (i < hi) {
+        for (int p = 0; p < parts; ++p) s += ldv<DT>(y, (t * parts + p) * (int64_t)width + i);
+        if (shared) s += sscale * ldv<DT>(shared, t * (int64_t)width + i);
+        if (gate) {
+          float r = ldv<DT>(gate, t * gate_ld + i);
+          if (gate_bias) r += ldv<DT>(gate_bias, i);
+          s *= sigmoid_f<EXACT>(r);
+        }
+      }
+      val[k] = s;
+      ss += s * s;
+    }
+    ss = block_sum256(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+    float s2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int i = lo + tid + 256 * k;
+      float v = 0.f;
+      if (i < hi) {
+        v = xr[i] + val[k] * inv * ldv<DT>(post_w, i);
+        xo[i] = v;
+      }
+      val[k] = v;
+      s2 += v * v;
+    }
+    s2 = block_sum256(s2, red);
+    if (h_out) {
+      const float inv2 = 1.0f / sqrtf(s2 / (float)gs + eps);
+#pragma unroll
+      for (int k = 0; k < NV; ++k) {
+        const int i = lo + tid + 256 * k;
+        if (i < hi) stv<DT>(h_out, t * (int64_t)width + i, val[k] * inv2 * ldv<DT>(next_w, i));
+      }
+    }
+  }
+}
+
+// out[t][j] = act(gate[t][j]) * up[t][j]; gate and up rows have their own strides (two column ranges of one projection, or two
+// tensors).  kind 0: silu, 1: gelu (tanh form), 2: sigmoid
+template <int DT>
+__global__ __launch_bounds__(256) void glu_act_kernel(void* __restrict__ out, const void* __restrict__ gate, int64_t gate_ld,
+                                                      const void* __restrict__ up, int64_t up_ld, int64_t n, int ff, int kind) {
+  constexpr bool EXACT = DT == LL_F32;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n * ff) return;
+  const int64_t t = idx / ff;
+  const int j = (int)(idx - t * ff);
+  const float g = ldv<DT>(gate, t * gate_ld + j), u = ldv<DT>(up, t * up_ld + j);
+  float a;
+  if (kind == 0) {
+    a = g * sigmoid_f<EXACT>(g);
+  } else if (kind == 2) {
+    a = sigmoid_f<EXACT>(g);
+  } else {
+    const float inner = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    // tanh(v) = 2 sigmoid(2 v) - 1: the 16-bit form takes the hardware exponential
+    const float th = EXACT ? tanhf(inner) : 2.0f * ll_sigmoidf(2.0f * inner) - 1.0f;
+    a = 0.5f * g * (1.0f + th);
+  }
+  stv<DT>(out, idx, a * u);
+}
+
+// logits <- cap tanh(logits / cap), fp32 arithmetic
+template <int DT>
+__global__ __launch_bounds__(256) void softcap_kernel(void* __restrict__ x, int64_t n, float cap) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  stv<DT>(x, idx, cap * tanhf(ldv<DT>(x, idx) / cap));
+}
+
+}  // namespace
+
+#define LL_BY_DTYPE(dtype, CALL)             \
+  do {                                       \
+    if (dtype == LL_F16) { CALL(LL_F16); }   \
+    else if (dtype == LL_BF16) { CALL(LL_BF16); } \
+    else { CALL(LL_F32); }                   \
+  } while (0)
+
+extern "C" int ll_gated_group_norm(const float* x_in, float* x_out, void* h_out, const void* y, int64_t parts, const void* shared,
+                                   const float* shared_scale, const void* gate, int64_t gate_ld, const void* gate_bias,
+                                   const void* post_w, const void* next_w, int64_t n, int64_t width, int64_t groups, float eps,
+                                   int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || width < 1 || width > (1 << 20) || groups < 1 || width % groups || parts < 0 || parts > 64) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!x_in) return LL_ERR_ARG;
+  if (y && (!x_out || !post_w || parts < 1)) return LL_ERR_ARG;
+  if (!y && (!h_out || shared || gate)) return LL_ERR_ARG;
+  if (h_out && !next_w) return LL_ERR_ARG;
+  if (shared && !shared_scale) return LL_ERR_ARG;
+  if (gate && gate_ld < width) return LL_ERR_SHAPE;
+  if (!y) x_out = const_cast<float*>(x_in);
+  const dim3 grid((unsigned)n);
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t gs = width / groups;
+#define LL_GN_ARGS \
+  x_in, x_out, h_out, y, (int)parts, shared, shared_scale, gate, gate_ld, gate_bias, post_w, next_w, (int)width, (int)groups, eps
+#define CALL(DT)                                                                                          \
+  if (y && gs <= 256) gated_group_norm_cached_kernel<DT, 1><<<grid, 256, 0, st>>>(LL_GN_ARGS);            \
+  else if (y && gs <= 1024) gated_group_norm_cached_kernel<DT, 4><<<grid, 256, 0, st>>>(LL_GN_ARGS);      \
+  else if (y && gs <= 4096) gated_group_norm_cached_kernel<DT, 16><<<grid, 256, 0, st>>>(LL_GN_ARGS);     \
+  else gated_group_norm_kernel<DT><<<grid, 256, 0, st>>>(LL_GN_ARGS)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+#undef LL_GN_ARGS
+  return LL_LAUNCH_CHECK();
+}
+
+extern "C" int ll_glu_act(void* out, const void* gate, int64_t gate_ld, const void* up, int64_t up_ld, int64_t n, int64_t ff,
+                          int kind, int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || ff < 1 || gate_ld < ff || up_ld < ff || ff > (1 << 24) || kind < 0 || kind > 2) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!out || !gate || !up) return LL_ERR_ARG;
+  const dim3 grid((unsigned)((n * ff + 255) / 256));
+  hipStream_t st = (hipStream_t)stream;
+#define CALL(DT) glu_act_kernel<DT><<<grid, 256, 0, st>>>(out, gate, gate_ld, up, up_ld, n, (int)ff, kind)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+  return LL_LAUNCH_CHECK();
+}
+
+extern "C" int ll_softcap(void* x, int64_t n, float cap, int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || !(cap > 0.f)) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!x) return LL_ERR_ARG;
+  const dim3 grid((unsigned)((n + 255) / 256));
+  hipStream_t st = (hipStream_t)stream;
+#define CALL(DT) softcap_kernel<DT><<<grid, 256, 0, st>>>(x, n, cap)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+  return LL_LAUNCH_CHECK();
+}

@@ -184,7 +184,7 @@ __global__ __launch_bounds__(256) void ragged_attention_kernel(
     const void* __restrict__ q, const void* __restrict__ k_cache, const void* __restrict__ v_cache,
     const int32_t* __restrict__ token_table, int64_t tt_stride, const int32_t* __restrict__ seq_req,
     const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const void* __restrict__ sink, float scale,
-    void* __restrict__ out, int64_t n, int heads, int kv_heads, int dk, int dv) {
+    void* __restrict__ out, int64_t n, int heads, int kv_heads, int dk, int dv, int64_t k_stride, int64_t v_stride, int window) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   float* sq = lds + wave * (dk + 128);  // [dk] query
@@ -196,7 +196,9 @@ __global__ __launch_bounds__(256) void ragged_attention_kernel(
   const int h = (int)(w - t * heads);
   const int g = h / (heads / kv_heads);
   const int pos = tok_pos[t];
-  const bool vec = (dk % (DT == LL_F32 ? 4 : 8) == 0) && ((reinterpret_cast<uintptr_t>(k_cache) & 15u) == 0);
+  const bool vec = (dk % (DT == LL_F32 ? 4 : 8) == 0) && (k_stride % (DT == LL_F32 ? 4 : 8) == 0) &&
+                   ((reinterpret_cast<uintptr_t>(k_cache) & 15u) == 0);
+  const int first_key = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;   // a window keeps the last `window` keys
   const int32_t* table = token_table + (int64_t)seq_req[tok_seq[t]] * tt_stride;
   for (int c = lane; c < dk; c += 64) sq[c] = ldv<DT>(q, (t * heads + h) * dk + c);
   float m = -INFINITY, l = 0.f;
@@ -208,13 +210,13 @@ __global__ __launch_bounds__(256) void ragged_attention_kernel(
 #pragma unroll
   for (int i = 0; i < VPL; ++i) acc[i] = 0.f;
   __builtin_amdgcn_wave_barrier();
-  for (int base = 0; base <= pos; base += 64) {
+  for (int base = first_key; base <= pos; base += 64) {
     const int j = base + lane;
     float s = -INFINITY;
     int row = 0;
     if (j <= pos) {
       row = table[j];
-      const int64_t kb = ((int64_t)row * kv_heads + g) * dk;
+      const int64_t kb = (int64_t)row * k_stride + (int64_t)g * dk;
       s = dot_row<DT>(sq, k_cache, kb, dk, vec) * scale;
     }
     const float tile_max = wave_max(s);
@@ -232,7 +234,7 @@ __global__ __launch_bounds__(256) void ragged_attention_kernel(
       const int c = lane + 64 * i;
       float a = acc[i] * corr;
       if (c < dv) {
-        for (int jj = 0; jj < cnt; ++jj) a += sp[jj] * ldv<DT>(v_cache, ((int64_t)sr[jj] * kv_heads + g) * dv + c);
+        for (int jj = 0; jj < cnt; ++jj) a += sp[jj] * ldv<DT>(v_cache, (int64_t)sr[jj] * v_stride + (int64_t)g * dv + c);
       }
       acc[i] = a;
     }
@@ -284,9 +286,11 @@ extern "C" int ll_qk_norm_cache(const void* qkv, int64_t ld, const void* q_w, co
 extern "C" int ll_ragged_attention(const void* q, const void* k_cache, const void* v_cache, const int32_t* token_table,
                                    int64_t tt_stride, const int32_t* seq_req, const int32_t* tok_seq, const int32_t* tok_pos,
                                    const void* sink, float scale, void* out, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk,
-                                   int64_t dv, int dtype, void* stream) {
+                                   int64_t dv, int64_t k_stride, int64_t v_stride, int64_t window, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
-  if (n < 0 || heads < 1 || kv_heads < 1 || heads % kv_heads || dk < 1 || dk > 1024 || dv < 1 || dv > 256) return LL_ERR_SHAPE;
+  if (n < 0 || heads < 1 || kv_heads < 1 || heads % kv_heads || dk < 1 || dk > 1024 || dv < 1 || dv > 1024 || window < 0 ||
+      window > 0x7fffffff || k_stride < kv_heads * dk || v_stride < kv_heads * dv)
+    return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
   if (!q || !k_cache || !v_cache || !token_table || !seq_req || !tok_seq || !tok_pos || !out) return LL_ERR_ARG;
   const int64_t waves = n * heads;
@@ -296,11 +300,14 @@ extern "C" int ll_ragged_attention(const void* q, const void* k_cache, const voi
   hipStream_t st = (hipStream_t)stream;
 #define CALL_V(DT, V)                                                                                                        \
   ragged_attention_kernel<DT, V><<<grid, 256, lds, st>>>(q, k_cache, v_cache, token_table, tt_stride, seq_req, tok_seq, tok_pos, \
-                                                         sink, scale, out, n, (int)heads, (int)kv_heads, (int)dk, (int)dv)
+                                                         sink, scale, out, n, (int)heads, (int)kv_heads, (int)dk, (int)dv, k_stride, \
+                                                         v_stride, (int)window)
 #define CALL(DT)                     \
   if (vpl == 1) CALL_V(DT, 1);       \
   else if (vpl == 2) CALL_V(DT, 2);  \
-  else CALL_V(DT, 4)
+  else if (vpl <= 4) CALL_V(DT, 4);  \
+  else if (vpl <= 8) CALL_V(DT, 8);  \
+  else CALL_V(DT, 16)
   LL_BY_DTYPE(dtype, CALL);
 #undef CALL
 #undef CALL_V

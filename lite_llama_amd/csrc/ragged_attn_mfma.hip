@@ -49,7 +49,7 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
     const int32_t* __restrict__ token_table, int64_t tt_stride, const int32_t* __restrict__ seq_req,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const uint16_t* __restrict__ sink,
     float scale_log2, uint16_t* __restrict__ out, float* __restrict__ partials, int max_parts, int heads, int kv_heads, int dk,
-    int dv) {
+    int dv, int64_t k_stride, int64_t v_stride, int window) {
   constexpr int QB = 1;
   constexpr bool DECODE = true;
   constexpr int VSTR = NTM * 16 + 8;
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
   const int b = blockIdx.z;
   const int start = seq_start[b], first = seq_first_pos[b];
   const int group = heads / kv_heads;
-  int g, k_lo, k_hi;
+  int g, k_lo, k_hi, k_begin;   // k_begin: the first key a window still keeps (0 without one)
   int head[QB], token[QB], qpos[QB];
   bool valid[QB];
   {
@@ -69,9 +69,11 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
     head[0] = g * group + (valid[0] ? h0 + t : h0);
     token[0] = start;
     qpos[0] = first;  // (a decoded token: the sequence brings one)
+    k_begin = window > 0 && first - window + 1 > 0 ? first - window + 1 : 0;
     k_lo = blockIdx.x * kPart;
-    if (k_lo > first) return;
+    if (k_lo > first || k_lo + kPart <= k_begin) return;   // (a partition past the token, or wholly in front of the window)
     k_hi = k_lo + kPart < first + 1 ? k_lo + kPart : first + 1;
+    if (k_lo < k_begin) k_lo = (k_begin / 32) * 32;         // the window's first partition starts at the tile that holds k_begin
   }
   const int32_t* table = token_table + (int64_t)seq_req[b] * tt_stride;
   const uint16_t* vtr = lds_v + (4 * c + (t >> 2)) * VSTR + (t & 3) * 4;
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
     }
     m_i[qb] = -INFINITY;
     d_i[qb] = 0.f;
-    if (sink && k_lo == 0) {
+    if (sink && (int)blockIdx.x == k_begin / kPart) {
       m_i[qb] = to_f32<DT>(sink[head[qb]]) * kLog2e;
       d_i[qb] = 1.0f;
     }
@@ -108,10 +110,10 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
   };
   auto fetch = [&](int p, int64_t ra, int64_t rb, Q4 (&fa)[NSM], Q4 (&fb)[NSM], Q4 (&ga)[NTM / 2], Q4 (&gb)[NTM / 2]) {
     const bool okA = p + t < k_hi, okB = p + 16 + t < k_hi;
-    const uint16_t* kA = k_cache + (ra * kv_heads + g) * dk;
-    const uint16_t* kB = k_cache + (rb * kv_heads + g) * dk;
-    const uint16_t* vA = v_cache + (ra * kv_heads + g) * dv;
-    const uint16_t* vB = v_cache + (rb * kv_heads + g) * dv;
+    const uint16_t* kA = k_cache + ra * k_stride + (int64_t)g * dk;
+    const uint16_t* kB = k_cache + rb * k_stride + (int64_t)g * dk;
+    const uint16_t* vA = v_cache + ra * v_stride + (int64_t)g * dv;
+    const uint16_t* vB = v_cache + rb * v_stride + (int64_t)g * dv;
 #pragma unroll
     for (int s = 0; s < NSM; ++s) {
       const int ch = 8 * (4 * s + c);
@@ -157,12 +159,13 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int k0i = p0 + 4 * c + r, k1i = k0i + 16;
-        sc[r] = (k0i <= qpos[qb] && k0i < k_hi) ? sa[r] * scale_log2 : -INFINITY;
-        sc[4 + r] = (k1i <= qpos[qb] && k1i < k_hi) ? sb[r] * scale_log2 : -INFINITY;
+        sc[r] = (k0i <= qpos[qb] && k0i < k_hi && k0i >= k_begin) ? sa[r] * scale_log2 : -INFINITY;
+        sc[4 + r] = (k1i <= qpos[qb] && k1i < k_hi && k1i >= k_begin) ? sb[r] * scale_log2 : -INFINITY;
         mx = fmaxf(mx, fmaxf(sc[r], sc[4 + r]));
       }
       mx = rows_max(mx);
-      const float m_new = fmaxf(m_i[qb], mx);   // finite: the first key of the range is visible to every column
+      float m_new = fmaxf(m_i[qb], mx);
+      if (m_new == -INFINITY) m_new = 0.f;      // nothing seen yet and nothing visible in this tile: every weight is exp2(-inf) = 0
       alpha[qb] = m_i[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_i[qb] - m_new);
       float p[8];
       float ps = 0.f;
@@ -173,7 +176,7 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
       }
       ps = rows_sum(ps);
       d_i[qb] = d_i[qb] * alpha[qb] + ps;
-      m_i[qb] = m_new;
+      m_i[qb] = fmaxf(m_i[qb], mx);
       moved[qb] = __builtin_amdgcn_ballot_w64(alpha[qb] != 1.0f) != 0;
       uint16_t hi[8], lo[8];
 #pragma unroll
@@ -272,7 +275,8 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     const int32_t* __restrict__ token_table, int64_t tt_stride, const int32_t* __restrict__ seq_req,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const uint16_t* __restrict__ sink,
-    float scale_log2, uint16_t* __restrict__ out, int heads, int kv_heads, int dk, int dv) {
+    float scale_log2, uint16_t* __restrict__ out, int heads, int kv_heads, int dk, int dv, int64_t k_stride, int64_t v_stride,
+    int window) {
   constexpr int KSTR = NSM * 32 + 8, VSTR = NTM * 16 + 8;
   constexpr int KPASS = (32 * NSM * 4 + 255) / 256, VPASS = (32 * NTM * 2 + 255) / 256;  // 16-byte pieces per thread
   __shared__ __attribute__((aligned(16))) uint16_t lds_k[32 * KSTR];
@@ -290,6 +294,11 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
   const int token = start + qi, qpos = first + qi;
   const int k_hi = first + (q0 + 64 < count ? q0 + 64 : count);            // the workgroup's key range
   const int k_hi_w = first + (qw + 16 < count ? qw + 16 : count);         // this wave's
+  // with a window a column at position p sees keys p - window + 1 .. p: the workgroup starts at the tile that holds the first
+  // key of its first column, a wave skips tiles in front of its own first column's window
+  const int k_lo_wg = window > 0 && first + q0 - window + 1 > 0 ? ((first + q0 - window + 1) / 32) * 32 : 0;
+  const int k_lo_w = window > 0 && first + qw - window + 1 > 0 ? first + qw - window + 1 : 0;
+  const int wlo = window > 0 ? qpos - window + 1 : 0;
   const int32_t* table = token_table + (int64_t)seq_req[b] * tt_stride;
   const int ns = (dk + 31) / 32, nt = (dv + 15) / 16;
   const int kcpr = dk / 8, vcpr = dv / 8;                                  // 16-byte pieces per cache row
@@ -319,13 +328,13 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
   _Pragma("unroll") for (int u = 0; u < KPASS; ++u) {                                                              \
     const int i = tid + 256 * u, key = i / kcpr, piece = i - key * kcpr;                                           \
     kr[u] = (key < 32 && (P) + key < k_hi)                                                                         \
-                ? *reinterpret_cast<const Q4*>(k_cache + ((int64_t)table[(P) + key] * kv_heads + g) * dk + 8 * piece) \
+                ? *reinterpret_cast<const Q4*>(k_cache + (int64_t)table[(P) + key] * k_stride + (int64_t)g * dk + 8 * piece) \
                 : Q4{0, 0, 0, 0};                                                                                  \
   }                                                                                                                \
   _Pragma("unroll") for (int u = 0; u < VPASS; ++u) {                                                              \
     const int i = tid + 256 * u, key = i / vcpr, piece = i - key * vcpr;                                           \
     vr[u] = (key < 32 && (P) + key < k_hi)                                                                         \
-                ? *reinterpret_cast<const Q4*>(v_cache + ((int64_t)table[(P) + key] * kv_heads + g) * dv + 8 * piece) \
+                ? *reinterpret_cast<const Q4*>(v_cache + (int64_t)table[(P) + key] * v_stride + (int64_t)g * dv + 8 * piece) \
                 : Q4{0, 0, 0, 0};                                                                                  \
   }
 #define LL_STAGE()                                                                           \
@@ -337,13 +346,13 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
     const int i = tid + 256 * u, key = i / vcpr, piece = i - key * vcpr;                     \
     if (key < 32) *reinterpret_cast<Q4*>(&lds_v[key * VSTR + 8 * piece]) = vr[u];            \
   }
-  LL_FETCH(0)
+  LL_FETCH(k_lo_wg)
   __syncthreads();   // the zero fill is complete
   LL_STAGE()
   __syncthreads();
-  for (int p0 = 0; p0 < k_hi; p0 += 32) {
+  for (int p0 = k_lo_wg; p0 < k_hi; p0 += 32) {
     if (p0 + 32 < k_hi) { LL_FETCH(p0 + 32) }
-    if (wave_on && p0 < k_hi_w) {
+    if (wave_on && p0 < k_hi_w && p0 + 32 > k_lo_w) {
       f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < NSM; ++s) {
@@ -359,12 +368,13 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int k0i = p0 + 4 * c + r, k1i = k0i + 16;
-        sc[r] = k0i <= qpos ? sa[r] * scale_log2 : -INFINITY;
-        sc[4 + r] = k1i <= qpos ? sb[r] * scale_log2 : -INFINITY;
+        sc[r] = (k0i <= qpos && k0i >= wlo) ? sa[r] * scale_log2 : -INFINITY;
+        sc[4 + r] = (k1i <= qpos && k1i >= wlo) ? sb[r] * scale_log2 : -INFINITY;
         mx = fmaxf(mx, fmaxf(sc[r], sc[4 + r]));
       }
       mx = rows_max(mx);
-      const float m_new = fmaxf(m_i, mx);   // finite: key 0 is visible to every column
+      float m_new = fmaxf(m_i, mx);
+      if (m_new == -INFINITY) m_new = 0.f;  // a column whose window starts behind this tile and that has seen nothing yet
       const float alpha = m_i == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_i - m_new);
       float ps = 0.f;
       uint16_t hi[8], lo[8];
@@ -376,7 +386,7 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
       }
       ps = rows_sum(ps);
       d_i = d_i * alpha + ps;
-      m_i = m_new;
+      m_i = fmaxf(m_i, mx);
       const Q4 pf_hi = {(uint32_t)hi[0] | ((uint32_t)hi[1] << 16), (uint32_t)hi[2] | ((uint32_t)hi[3] << 16),
                         (uint32_t)hi[4] | ((uint32_t)hi[5] << 16), (uint32_t)hi[6] | ((uint32_t)hi[7] << 16)};
       const Q4 pf_lo = {(uint32_t)lo[0] | ((uint32_t)lo[1] << 16), (uint32_t)lo[2] | ((uint32_t)lo[3] << 16),
@@ -425,20 +435,23 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
 template <int DT>
 __global__ __launch_bounds__(256) void ragged_attention_merge_kernel(const float* __restrict__ partials, int max_parts,
                                                                      const int32_t* __restrict__ seq_first_pos,
-                                                                     uint16_t* __restrict__ out, int64_t n, int heads, int dv) {
+                                                                     uint16_t* __restrict__ out, int64_t n, int heads, int dv,
+                                                                     int window) {
   const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (w >= n * heads) return;
   const int lane = threadIdx.x & 63;
   const int64_t token = w / heads;
-  const int parts = seq_first_pos[token] / kPart + 1;  // (decoded tokens: token index == sequence index)
+  const int pos = seq_first_pos[token];                // (decoded tokens: token index == sequence index)
+  const int parts = pos / kPart + 1;
+  const int p_lo = window > 0 && pos - window + 1 > 0 ? (pos - window + 1) / kPart : 0;   // partitions in front of it wrote nothing
   const float* src = partials + w * max_parts * (2 + dv);
   float m = -INFINITY;
-  for (int p = 0; p < parts; ++p) m = fmaxf(m, src[p * (2 + dv)]);
+  for (int p = p_lo; p < parts; ++p) m = fmaxf(m, src[p * (2 + dv)]);
   float d = 0.f;
-  for (int p = 0; p < parts; ++p) d += src[p * (2 + dv) + 1] * exp2f(src[p * (2 + dv)] - m);
+  for (int p = p_lo; p < parts; ++p) d += src[p * (2 + dv) + 1] * exp2f(src[p * (2 + dv)] - m);
   for (int ch = lane; ch < dv; ch += 64) {
     float o = 0.f;
-    for (int p = 0; p < parts; ++p) o += src[p * (2 + dv) + 2 + ch] * exp2f(src[p * (2 + dv)] - m);
+    for (int p = p_lo; p < parts; ++p) o += src[p * (2 + dv) + 2 + ch] * exp2f(src[p * (2 + dv)] - m);
     out[w * dv + ch] = from_f32<DT>(o / d);
   }
 }
@@ -458,8 +471,12 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
                                         int64_t tt_stride, const int32_t* seq_req, const int32_t* seq_start,
                                         const int32_t* seq_first_pos, const void* sink, float scale, void* out, int64_t n,
                                         int64_t batch, int64_t longest_run, int64_t longest_context, int decode, float* partials,
-                                        int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int dtype, void* stream) {
+                                        int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int64_t k_stride, int64_t v_stride,
+                                        int64_t window, int dtype, void* stream) {
   if (!ll_ragged_attention_mfma_supported(dk, dv, dtype)) return dtype == LL_F32 ? LL_ERR_DTYPE : LL_ERR_SHAPE;
+  if (k_stride < kv_heads * dk || v_stride < kv_heads * dv || k_stride % 8 || v_stride % 8 || window < 0 || window > 0x7fffffff ||
+      !ll_aligned16(k_cache) || !ll_aligned16(v_cache) || !ll_aligned16(q))
+    return LL_ERR_SHAPE;
   if (n < 0 || batch < 0 || heads < 1 || kv_heads < 1 || heads % kv_heads || heads > 65535 || batch > 65535 || longest_run < 1 ||
       longest_context < 1 || (decode && n != batch))
     return LL_ERR_SHAPE;
@@ -475,7 +492,7 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
   ragged_attention_mfma_decode_kernel<DT, NS, NT><<<grid, 64, 0, st>>>(                                                      \
       (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, token_table, tt_stride, seq_req, seq_start,    \
       seq_first_pos, (const uint16_t*)sink, scale_log2, (uint16_t*)out, partials, max_parts, (int)heads, (int)kv_heads, (int)dk, \
-      (int)dv)
+      (int)dv, k_stride, v_stride, (int)window)
 #define CALL(DT)                                         \
   if (dk <= 64 && dv <= 64) { CALL_D(DT, 2, 4); }        \
   else if (dk <= 128 && dv <= 128) { CALL_D(DT, 4, 8); } \
@@ -485,7 +502,8 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
 #define CALL_4(DT, NS, NT)                                                                                                  \
   ragged_attention_mfma_prefill4_kernel<DT, NS, NT><<<grid4, 256, 0, st>>>(                                                 \
       (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, token_table, tt_stride, seq_req, seq_start,   \
-      seq_first_pos, (const uint16_t*)sink, scale_log2, (uint16_t*)out, (int)heads, (int)kv_heads, (int)dk, (int)dv)
+      seq_first_pos, (const uint16_t*)sink, scale_log2, (uint16_t*)out, (int)heads, (int)kv_heads, (int)dk, (int)dv, k_stride,   \
+      v_stride, (int)window)
 #define CALL_P(DT)                                       \
   if (dk <= 64 && dv <= 64) { CALL_4(DT, 2, 4); }        \
   else if (dk <= 128 && dv <= 128) { CALL_4(DT, 4, 8); } \
@@ -502,10 +520,10 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
     const int64_t waves = n * heads;
     if (dtype == LL_F16)
       ragged_attention_merge_kernel<LL_F16><<<dim3((unsigned)((waves + 3) / 4)), 256, 0, st>>>(partials, max_parts, seq_first_pos,
-                                                                                            (uint16_t*)out, n, (int)heads, (int)dv);
+                                                                                            (uint16_t*)out, n, (int)heads, (int)dv, (int)window);
     else
       ragged_attention_merge_kernel<LL_BF16><<<dim3((unsigned)((waves + 3) / 4)), 256, 0, st>>>(partials, max_parts, seq_first_pos,
-                                                                                             (uint16_t*)out, n, (int)heads, (int)dv);
+                                                                                             (uint16_t*)out, n, (int)heads, (int)dv, (int)window);
   }
   return LL_LAUNCH_CHECK();
 }

@@ -7,6 +7,8 @@
 //   ll_cast_pair / ll_residual_set   the two ends of a projection over [x ; x0] that re-enters the residual stream
 //   ll_gated_linear_scan   per-head linear recurrence S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, o_t = S_t^T q_t with a
 //                          lower-bounded forget gate and a per-head RMS norm of o (HGRN2), state in fp32 slots
+//   ll_mingru_scan         per-channel gated recurrence S_t = (1 - z_t) S_(t-1) + z_t c_t whose gates read the current token
+//                          only (minGRU), silu-gated read-out, state in fp32 slots
 //
 // Storage dtype DT = LL_F16 / LL_BF16 / LL_F32 for activations and weights; everything that the recurrence, the norms and
 // the residual touch is fp32.  A step is described by   seq_start[b + 1] (first flat token of each sequence's run),
@@ -495,6 +497,51 @@ inline unsigned flat_grid(int64_t total) {
   return (unsigned)(g < 1 ? 1 : (g > (1 << 20) ? (1 << 20) : g));  // (one piece per thread up to 2^28 pieces: no ragged second pass)
 }
 
+// minGRU: S_t = (1 - z_t) S_(t-1) + z_t c_t per channel, with z = sigmoid(z_raw + z_bias), u = x_raw + x_bias and the candidate
+// c = u + 1/2 for u >= 0, sigmoid(u) below; the read-out is S_t * silu(g_raw).  Rows hold [z_raw | x_raw | g_raw] (stride ld).
+// One thread per (sequence, channel) walks the run's tokens in order; neighbouring threads read neighbouring channels.  The
+// loads of four tokens are issued before the four dependent state updates.  State fp32 [slots][width].
+template <int DT>
+__global__ __launch_bounds__(256) void mingru_scan_kernel(const void* __restrict__ z, const void* __restrict__ x,
+                                                          const void* __restrict__ g, int64_t ld, const void* __restrict__ z_bias,
+                                                          const void* __restrict__ x_bias, void* __restrict__ out, int width,
+                                                          const int32_t* __restrict__ seq_start,
+                                                          const int32_t* __restrict__ seq_first_pos,
+                                                          const int32_t* __restrict__ seq_slot, float* __restrict__ state) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= width) return;
+  const int b = blockIdx.y;
+  const int start = seq_start[b], stop = seq_start[b + 1];
+  float* slot = state + (int64_t)seq_slot[b] * width + c;
+  float S = seq_first_pos[b] > 0 ? *slot : 0.f;
+  const float zb = z_bias ? ldv<DT>(z_bias, c) : 0.f, xb = x_bias ? ldv<DT>(x_bias, c) : 0.f;
+  auto update = [&](float zr, float xr, float gr, int64_t t) {
+    const float zt = 1.0f / (1.0f + expf(-(zr + zb)));
+    const float u = xr + xb;
+    const float cand = u >= 0.f ? u + 0.5f : 1.0f / (1.0f + expf(-u));
+    S = (1.0f - zt) * S + zt * cand;
+    stv<DT>(out, t * width + c, S * (gr / (1.0f + expf(-gr))));
+  };
+  int t = start;
+  for (; t + 4 <= stop; t += 4) {
+    float zr[4], xr[4], gr[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int64_t at = (int64_t)(t + k) * ld + c;
+      zr[k] = ldv<DT>(z, at);
+      xr[k] = ldv<DT>(x, at);
+      gr[k] = ldv<DT>(g, at);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) update(zr[k], xr[k], gr[k], t + k);
+  }
+  for (; t < stop; ++t) {
+    const int64_t at = (int64_t)t * ld + c;
+    update(ldv<DT>(z, at), ldv<DT>(x, at), ldv<DT>(g, at), t);
+  }
+  *slot = S;
+}
+
 }  // namespace
 
 #define LL_BY_DTYPE(dtype, CALL)             \
@@ -628,5 +675,21 @@ extern "C" int ll_gated_linear_scan(const void* q, const void* f, const void* v,
   LL_BY_DTYPE(dtype, CALL);
 #undef CALL
 #undef CALL_R
+  return LL_LAUNCH_CHECK();
+}
+
+extern "C" int ll_mingru_scan(const void* z, const void* x, const void* g, int64_t ld, const void* z_bias, const void* x_bias,
+                              void* out, int64_t batch, int64_t width, const int32_t* seq_start, const int32_t* seq_first_pos,
+                              const int32_t* seq_slot, float* state, int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (batch < 0 || batch > 65535 || width < 1 || ld < width) return LL_ERR_SHAPE;
+  if (batch == 0) return LL_OK;
+  if (!z || !x || !g || !out || !seq_start || !seq_first_pos || !seq_slot || !state) return LL_ERR_ARG;
+  const dim3 grid((unsigned)((width + 255) / 256), (unsigned)batch);
+  hipStream_t st = (hipStream_t)stream;
+#define CALL(DT) \
+  mingru_scan_kernel<DT><<<grid, 256, 0, st>>>(z, x, g, ld, z_bias, x_bias, out, (int)width, seq_start, seq_first_pos, seq_slot, state)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
   return LL_LAUNCH_CHECK();
 }

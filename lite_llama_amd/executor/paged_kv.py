@@ -96,15 +96,15 @@ class PagedKVPool:
 class PagedStateCache(PagedKVPool):
     """Cache of a model whose layer RUNS differ in what they keep per sequence (a layer that runs several times in a forward
     pass keeps one set per run): attention runs own ``(K [rows, kv_heads, dk], V [rows, kv_heads, dv])`` in the block pool --
-    key and value widths may differ --, recurrent runs own a fixed-size fp32 state ``[slots, heads, dk, dv]``, and any run may
+    key and value widths may differ --, latent-attention runs one row ``[latent | rotated key part]`` per token, recurrent runs own a fixed-size fp32 state ``[slots, heads, dk, dv]``, and any run may
     own a token-shift row pair ``[2, slots, width]`` (double-buffered by the sequence's parity).  One block allocator, one
     block table and one per-token row table serve all attention runs; a sequence's slot is its row of those tables, so blocks
     and slots are handed out and given back together.  Fixed-size state is never cleared: the kernels start a sequence whose
     run begins at position 0 from zeros, whatever an earlier owner of the slot left."""
 
     def __init__(self, runs, num_blocks: int, block_size: int, device, max_requests: int, max_seq_len: int, dtype):
-        """``runs``: one mapping per layer run: ``{"kind": "attention", "kv_heads", "dk", "dv"}`` or
-        ``{"kind": "recurrent", "heads", "dk", "dv"}``, each with an optional ``"shift_width"``."""
+        """``runs``: one mapping per layer run: ``{"kind": "attention", "kv_heads", "dk", "dv"}``, ``{"kind": "latent", "rank",
+        "rot"}`` or ``{"kind": "recurrent", "heads", "dk", "dv"}``, each with an optional ``"shift_width"``."""
         self.runs = [dict(r) for r in runs]
         self.dtype = dtype
         super().__init__(len(self.runs), num_blocks, block_size, 1, 1, device, max_requests, max_seq_len, dtype)
@@ -117,6 +117,12 @@ class PagedStateCache(PagedKVPool):
             if r["kind"] == "attention":
                 buffers.append((torch.zeros(self.max_tokens, r["kv_heads"], r["dk"], dtype=dtype, device=dev),
                                 torch.zeros(self.max_tokens, r["kv_heads"], r["dv"], dtype=dtype, device=dev)))
+                self.recurrent.append(None)
+            elif r["kind"] == "latent":
+                # one row [latent (rank) | rotated key part (rot)] per token: the keys of ONE key/value head; the values are the
+                # latent columns of the same rows (a row-strided view, nothing is stored twice)
+                rows = torch.zeros(self.max_tokens, 1, r["rank"] + r["rot"], dtype=dtype, device=dev)
+                buffers.append((rows, rows[:, :, :r["rank"]]))
                 self.recurrent.append(None)
             elif r["kind"] == "recurrent":
                 buffers.append(None)
@@ -133,10 +139,11 @@ class PagedStateCache(PagedKVPool):
         return self._extend(req_idx, new_lens, 0, longest_run, 1, token_table).view(req_idx.numel(), longest_run)
 
     def state_bytes(self) -> int:
-        total = 0
+        total, seen = 0, set()
         for group in (self.kv_buffer, self.recurrent, self.shift):
             for t in group:
                 for u in (t if isinstance(t, tuple) else (t,)):
-                    if u is not None:
-                        total += u.numel() * u.element_size()
+                    if u is not None and u.untyped_storage().data_ptr() not in seen:   # (a view of counted rows adds nothing)
+                        seen.add(u.untyped_storage().data_ptr())
+                        total += u.untyped_storage().nbytes()
         return total

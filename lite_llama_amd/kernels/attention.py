@@ -310,26 +310,32 @@ def qk_norm_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, q_weight, k_
 
 
 @torch.no_grad()
-def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=None):
+def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=None, window: int = 0):
     """Causal softmax attention of every token of a ragged step against positions ``0 .. its own`` of its sequence, keys and
-    values read through ``token_table[request][position]``; ``sink [heads]`` adds ``exp(sink_h)`` to each head's denominator.
-    Scores, weights and the output sum are fp32.  Returns ``[n, heads * dv]``."""
+    values read through ``token_table[request][position]``; ``sink [heads]`` adds ``exp(sink_h)`` to each head's denominator;
+    ``window > 0`` keeps the last ``window`` positions (the token's own included).  ``k_cache [rows, kv_heads, dk]`` /
+    ``v_cache [rows, kv_heads, dv]`` may be row-strided views (the values of a latent cache are a column range of its key
+    rows).  Scores, weights and the output sum are fp32.  Returns ``[n, heads * dv]``."""
     L.require_cuda(q, k_cache, v_cache, token_table)
     n, heads, dk = q.shape
     kv_heads, dv = v_cache.shape[1], v_cache.shape[2]
     dt = q.dtype
-    if not q.is_contiguous() or k_cache.dtype != dt or v_cache.dtype != dt or k_cache.shape[1:] != (kv_heads, dk) \
-            or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+    if not q.is_contiguous() or k_cache.dtype != dt or v_cache.dtype != dt or k_cache.shape[1:] != (kv_heads, dk):
         raise ValueError("ragged_attention: q [n, heads, dk], caches [rows, kv_heads, dk] / [rows, kv_heads, dv], one dtype")
+    for c, w in ((k_cache, dk), (v_cache, dv)):
+        if c.stride(2) != 1 or (kv_heads > 1 and c.stride(1) != w) or c.stride(0) < kv_heads * w:
+            raise ValueError("ragged_attention: cache rows hold their heads densely (only the row stride is free)")
     if token_table.dtype != torch.int32 or token_table.stride(1) != 1:
         raise ValueError("ragged_attention: the token table is row-major int32")
     if sink is not None and (sink.dtype != dt or sink.numel() != heads or not sink.is_contiguous()):
         raise ValueError("ragged_attention: sink is [heads] in the queries' dtype")
     if step.num_tokens != n:
         raise ValueError("ragged_attention: the step describes another number of tokens")
+    ks, vs = k_cache.stride(0), v_cache.stride(0)
     out = torch.empty(n, heads * dv, dtype=dt, device=q.device)
     if (step.longest_run and step.longest_context and L.has("ll_ragged_attention_mfma") and not os.environ.get("LL_RAGGED_ATTN_VALU")
-            and L.lib().ll_ragged_attention_mfma_supported(dk, dv, L.dtype_code(dt))):
+            and L.lib().ll_ragged_attention_mfma_supported(dk, dv, L.dtype_code(dt)) and ks % 8 == 0 and vs % 8 == 0
+            and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0):
         # 16-bit storage: the MFMA form -- tokens of a run as the columns of a wave (prompt portions, mixed steps), or, when every
         # sequence brings one decoded token, the query heads of a key/value head, with the context cut into partitions
         decode = step.longest_run == 1
@@ -339,10 +345,54 @@ def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), token_table.data_ptr(), token_table.stride(0),
             step.seq_req.data_ptr(), step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(), L.ptr(sink), float(scale),
             out.data_ptr(), n, step.num_seqs, step.longest_run, step.longest_context, 1 if decode else 0, L.ptr(scratch), heads,
-            kv_heads, dk, dv, L.dtype_code(dt), L.stream_ptr()), "ragged_attention_mfma")
+            kv_heads, dk, dv, ks, vs, int(window), L.dtype_code(dt), L.stream_ptr()), "ragged_attention_mfma")
         return out
     L.check(L.lib().ll_ragged_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), token_table.data_ptr(),
                                         token_table.stride(0), step.seq_req.data_ptr(), step.tok_seq.data_ptr(),
                                         step.tok_pos.data_ptr(), L.ptr(sink), float(scale), out.data_ptr(), n, heads, kv_heads, dk,
-                                        dv, L.dtype_code(dt), L.stream_ptr()), "ragged_attention")
+                                        dv, ks, vs, int(window), L.dtype_code(dt), L.stream_ptr()), "ragged_attention")
+    return out
+
+
+# ------------------------------------------------------------------------------------- #
+# attention over a shared latent (csrc/latent_attn.hip): what surrounds the projections
+# ------------------------------------------------------------------------------------- #
+@torch.no_grad()
+def latent_kv_prep(rows, kv_off: int, rank: int, rot: int, kv_norm_weight, eps: float, freq, pairs: int, amp: float, step, cache,
+                   q_off: int = 0, q_rank: int = 0, q_norm_weight=None):
+    """Rows of the fused input projection hold the key/value latent ``[rank]`` followed by the shared rotated key part
+    ``[rot]`` at column ``kv_off``: the cache rows ``step.select`` of ``cache [rows, rank + rot]`` receive
+    ``[RMS norm(latent) * weight | key part rotated at the token's position]``.  With ``q_rank`` the columns
+    ``q_off .. q_off + q_rank`` (a query latent) are RMS-normed with ``q_norm_weight`` and returned ``[n, q_rank]``.
+    ``freq`` fp32 ``[pairs]``: angle per position of pair i (entries 2i, 2i + 1); cos and sin are multiplied by ``amp``."""
+    L.require_cuda(rows, cache, freq, kv_norm_weight)
+    n, dt = rows.shape[0], rows.dtype
+    if rows.dim() != 2 or rows.stride(1) != 1 or cache.dim() != 2 or cache.stride(1) != 1 or cache.dtype != dt \
+            or cache.shape[1] != rank + rot:
+        raise ValueError("latent_kv_prep: rows [n, ld] and cache [rows, rank + rot] in one dtype, unit inner strides")
+    if freq.dtype != torch.float32 or freq.numel() < pairs or not freq.is_contiguous() or step.num_tokens != n:
+        raise ValueError("latent_kv_prep: fp32 frequencies, one per rotated pair; a step of the rows' token count")
+    for w, size in ((kv_norm_weight, rank), (q_norm_weight, q_rank)):
+        if w is not None and (w.dtype != dt or w.numel() != size or not w.is_contiguous()):
+            raise ValueError("latent_kv_prep: norm weights in the rows' dtype, one entry per normed column")
+    q_out = torch.empty(n, q_rank, dtype=dt, device=rows.device) if q_rank else None
+    L.check(L.lib().ll_latent_kv_prep(rows.data_ptr(), rows.stride(0), int(kv_off), int(rank), int(rot), kv_norm_weight.data_ptr(),
+                                      float(eps), freq.data_ptr(), int(pairs), float(amp), step.tok_pos.data_ptr(),
+                                      step.select.data_ptr(), cache.data_ptr(), cache.stride(0), int(q_off), int(q_rank),
+                                      L.ptr(q_norm_weight), L.ptr(q_out), n, L.dtype_code(dt), L.stream_ptr()), "latent_kv_prep")
+    return q_out
+
+
+@torch.no_grad()
+def rotate_pairs(q, q_off: int, rot: int, freq, pairs: int, amp: float, step, out, out_off: int):
+    """``q [n, heads, w]`` (unit inner stride): the ``rot`` entries at ``q_off`` of every head, rotated pair by pair at the
+    token's position, land at ``out[n, heads, w'][..., out_off : out_off + rot]`` (``out`` contiguous)."""
+    L.require_cuda(q, out, freq)
+    n, heads = q.shape[0], q.shape[1]
+    if q.dim() != 3 or out.dim() != 3 or q.stride(2) != 1 or not out.is_contiguous() or out.shape[:2] != q.shape[:2] \
+            or out.dtype != q.dtype or q_off + rot > q.shape[2] or out_off + rot > out.shape[2] or step.num_tokens != n:
+        raise ValueError("rotate_pairs: q [n, heads, w] and a contiguous out [n, heads, w'] of one dtype")
+    L.check(L.lib().ll_rotate_pairs(q.data_ptr(), q.stride(0), q.stride(1), int(q_off), int(rot), freq.data_ptr(), int(pairs),
+                                    float(amp), step.tok_pos.data_ptr(), out.data_ptr(), out.shape[2], int(out_off), n, heads,
+                                    L.dtype_code(q.dtype), L.stream_ptr()), "rotate_pairs")
     return out

@@ -244,3 +244,69 @@ def moe_router(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, norm_topk
                                   x.stride(0), gate_weight.stride(0), int(top_k), 1 if norm_topk_prob else 0, L.dtype_code(x.dtype),
                                   int(align_block), *ptrs, L.stream_ptr()), "moe_router")
     return (w, ids, aligned) if align_block > 0 else (w, ids)
+
+
+# ------------------------------------------------------------------------------------- #
+# sigmoid router over expert groups + grouped expert products for 16-bit and 32-bit storage (csrc/moe_sparse.hip)
+# ------------------------------------------------------------------------------------- #
+@torch.no_grad()
+def group_router(h: torch.Tensor, router_weight: torch.Tensor, top: int, group_count: int = 1, group_keep: int = 1,
+                 route_scale: float = 1.0, extra_weight: torch.Tensor | None = None):
+    """``scores = sigmoid(router_weight h)`` in fp32 (``h`` in its storage dtype); the experts form ``group_count`` equal groups
+    of neighbours, a group's score is the sum of its two best, the best ``group_keep`` groups stay eligible; the ``top`` best
+    eligible experts are chosen.  Returns ``(ids int32 [n, top], weights fp32 [n, top], extra)``: weights = chosen scores /
+    (their sum + 1e-20) * ``route_scale``, slot k = the k-th best; ``extra`` fp32 ``[n]`` = ``sigmoid(extra_weight . h)`` when a
+    further weight row is given (the scale of a shared expert), else ``None``."""
+    L.require_cuda(h, router_weight, extra_weight)
+    n, width = h.shape
+    experts = router_weight.shape[0]
+    if h.stride(1) != 1 or router_weight.dtype != h.dtype or not router_weight.is_contiguous() or router_weight.shape[1] != width:
+        raise ValueError("group_router: h [n, width] and router weights [experts, width] of one dtype")
+    if extra_weight is not None and (extra_weight.dtype != h.dtype or extra_weight.numel() != width or not extra_weight.is_contiguous()):
+        raise ValueError("group_router: the extra row has one weight per channel")
+    ids = torch.empty(n, top, dtype=torch.int32, device=h.device)
+    weights = torch.empty(n, top, dtype=torch.float32, device=h.device)
+    extra = torch.empty(n, dtype=torch.float32, device=h.device) if extra_weight is not None else None
+    L.check(L.lib().ll_group_router(h.data_ptr(), h.stride(0), router_weight.data_ptr(), L.ptr(extra_weight), n, width, experts,
+                                    int(top), int(group_count), int(group_keep), float(route_scale), ids.data_ptr(),
+                                    weights.data_ptr(), L.ptr(extra), L.dtype_code(h.dtype), L.stream_ptr()), "group_router")
+    return ids, weights, extra
+
+
+@torch.no_grad()
+def sparse_glu_experts(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor,
+                       weights: torch.Tensor) -> torch.Tensor:
+    """Per slot (token, k): ``weights * down_e(silu(gate_e h) * up_e h)`` with ``e = ids[token, k]``; ``w_gate_up
+    [experts, 2 ff, width]`` (gate rows, then up rows), ``w_down [experts, width, ff]``.  Returns the slots' rows
+    ``[n, top, width]`` in the storage dtype (their sum over k is the caller's: the norm that follows adds them in fp32).
+    Slots are sorted by expert on the device; every product accumulates in fp32."""
+    L.require_cuda(h, w_gate_up, w_down, ids, weights)
+    n, width = h.shape
+    experts, two_ff, _ = w_gate_up.shape
+    ff, top = two_ff // 2, ids.shape[1]
+    dt = h.dtype
+    if (not h.is_contiguous() or w_gate_up.dtype != dt or w_down.dtype != dt or not w_gate_up.is_contiguous()
+            or not w_down.is_contiguous() or w_gate_up.shape[2] != width or tuple(w_down.shape) != (experts, width, ff)):
+        raise ValueError("sparse_glu_experts: h [n, width], gate|up [E, 2 ff, width], down [E, width, ff] of one dtype")
+    if ids.dtype != torch.int32 or weights.dtype != torch.float32 or not ids.is_contiguous() or not weights.is_contiguous() \
+            or weights.shape != ids.shape:
+        raise ValueError("sparse_glu_experts: int32 ids and fp32 weights [n, top]")
+    lib = L.lib()
+    block = int(lib.ll_moe_rows_block())
+    slots = n * top
+    padded = slots + experts * (block - 1)
+    meta = torch.empty(experts + padded + -(-padded // block) + 1, dtype=torch.int32, device=h.device)
+    counts, sorted_ids = meta[:experts], meta[experts:experts + padded]
+    block_expert, num_post = meta[experts + padded:-1], meta[-1:]
+    L.check(lib.ll_moe_sort(ids.data_ptr(), slots, experts, counts.data_ptr(), sorted_ids.data_ptr(), block_expert.data_ptr(),
+                            num_post.data_ptr(), L.stream_ptr()), "moe_sort")
+    act = torch.empty(slots, ff, dtype=dt, device=h.device)
+    out = torch.empty(n, top, width, dtype=dt, device=h.device)
+    code, st = L.dtype_code(dt), L.stream_ptr()
+    L.check(lib.ll_moe_rows_gemm(h.data_ptr(), h.stride(0), top, w_gate_up.data_ptr(), w_gate_up.stride(0), width, ff, 1, 0,
+                                 act.data_ptr(), ff, sorted_ids.data_ptr(), block_expert.data_ptr(), num_post.data_ptr(), slots,
+                                 experts, code, st), "moe_rows_gemm (gate|up)")
+    L.check(lib.ll_moe_rows_gemm(act.data_ptr(), ff, 1, w_down.data_ptr(), w_down.stride(0), ff, width, 0, weights.data_ptr(),
+                                 out.data_ptr(), width, sorted_ids.data_ptr(), block_expert.data_ptr(), num_post.data_ptr(), slots,
+                                 experts, code, st), "moe_rows_gemm (down)")
+    return out

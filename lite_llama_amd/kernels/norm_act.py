@@ -413,3 +413,91 @@ def residual_set(y: torch.Tensor, bias: torch.Tensor | None = None, out: torch.T
     L.check(L.lib().ll_residual_set(out.data_ptr(), y.data_ptr(), L.ptr(bias), n, width, L.dtype_code(y.dtype), L.stream_ptr()),
             "residual_set")
     return out
+
+
+# ------------------------------------------------------------------------------------- #
+# sublayers between two grouped norms, with a gate on the residual branch (csrc/group_norm.hip)
+# ------------------------------------------------------------------------------------- #
+class GatedUpdate:
+    """A sublayer's result that has not entered the residual stream yet: ``y [n, parts, width]`` (``parts`` rows per token
+    are summed: the experts a token chose), optionally ``+ shared_scale[t] * shared[t]``, times ``sigmoid(gate + gate_bias)``
+    (``gate``: a column range of a projection's rows), to be normed with ``post_weight`` and added."""
+
+    __slots__ = ("y", "shared", "shared_scale", "gate", "gate_bias", "post_weight")
+
+    def __init__(self, y, post_weight, gate=None, gate_bias=None, shared=None, shared_scale=None):
+        self.y = y if y.dim() == 3 else y.unsqueeze(1)
+        self.post_weight, self.gate, self.gate_bias, self.shared, self.shared_scale = post_weight, gate, gate_bias, shared, shared_scale
+
+    def rows(self, index: torch.Tensor) -> "GatedUpdate":
+        """The update of the listed tokens only."""
+        pick = lambda t: None if t is None else t[index].contiguous()  # noqa: E731
+        return GatedUpdate(pick(self.y), self.post_weight, pick(self.gate), self.gate_bias, pick(self.shared), pick(self.shared_scale))
+
+
+@torch.no_grad()
+def gated_group_norm(x: torch.Tensor, update: "GatedUpdate | None", next_weight, eps: float, groups: int = 1):
+    """``x`` (fp32 residual ``[n, width]``, updated IN PLACE): ``x += groupnorm(update) * post_weight`` -- the update's rows
+    summed, scaled by the sigmoid of its gate --, then ``h = groupnorm(x) * next_weight`` in the storage dtype
+    (``next_weight=None``: only the residual is updated).  ``groupnorm``: the row in ``groups`` equal consecutive parts, each
+    divided by ``sqrt(mean(part^2) + eps)``.  All sums, norms and the gate are fp32.  Returns ``h`` (or ``None``)."""
+    L.require_cuda(x, next_weight)
+    n, width = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or width % groups:
+        raise ValueError("gated_group_norm: a contiguous fp32 residual whose width the groups divide")
+    u = update
+    dt = (next_weight if next_weight is not None else u.post_weight).dtype
+    h = torch.empty(n, width, dtype=dt, device=x.device) if next_weight is not None else None
+    if next_weight is not None and (next_weight.numel() != width or not next_weight.is_contiguous()):
+        raise ValueError("gated_group_norm: the norm weight has one entry per channel")
+    args = (0, 0, 0, 0, 0, 0, 0, 0)
+    if u is not None:
+        if u.y.dtype != dt or u.y.shape[0] != n or u.y.shape[2] != width or not u.y.is_contiguous() or u.post_weight.dtype != dt:
+            raise ValueError("gated_group_norm: the update is [n, parts, width] in the weights' dtype")
+        gate_ld = 0
+        if u.gate is not None:
+            if u.gate.dtype != dt or u.gate.shape != (n, width) or u.gate.stride(1) != 1:
+                raise ValueError("gated_group_norm: gate logits are [n, width] with a unit inner stride")
+            gate_ld = u.gate.stride(0)
+        if u.shared is not None and (u.shared.dtype != dt or u.shared.shape != (n, width) or not u.shared.is_contiguous()
+                                     or u.shared_scale.dtype != torch.float32 or u.shared_scale.numel() != n):
+            raise ValueError("gated_group_norm: the shared row is [n, width], its scale fp32 [n]")
+        args = (u.y.data_ptr(), u.y.shape[1], L.ptr(u.shared), L.ptr(u.shared_scale), L.ptr(u.gate), gate_ld, L.ptr(u.gate_bias),
+                u.post_weight.data_ptr())
+    elif h is None:
+        return None
+    L.check(L.lib().ll_gated_group_norm(x.data_ptr(), x.data_ptr(), L.ptr(h), *args, L.ptr(next_weight), n, width, int(groups),
+                                        float(eps), L.dtype_code(dt), L.stream_ptr()), "gated_group_norm")
+    return h
+
+
+_GLU_KINDS = {"silu": 0, "gelu_tanh": 1, "sigmoid": 2}
+
+
+@torch.no_grad()
+def glu_act(gate: torch.Tensor, ff: int, kind: str, up: torch.Tensor | None = None) -> torch.Tensor:
+    """``act(gate[:, :ff]) * up[:, :ff]``; without ``up`` the rows of ``gate`` hold ``[gate | up]``.  Both may be wider,
+    row-strided views (column ranges of a fused projection).  ``kind``: ``"silu"``, ``"gelu_tanh"`` or ``"sigmoid"``.  fp32
+    arithmetic, one rounding to the storage dtype."""
+    if up is None:
+        if gate.shape[1] < 2 * ff:
+            raise ValueError("glu_act: rows hold [gate | up]")
+        up = gate[:, ff:]
+    L.require_cuda(gate, up)
+    if gate.dim() != 2 or up.dim() != 2 or gate.stride(1) != 1 or up.stride(1) != 1 or gate.shape[1] < ff or up.shape[1] < ff \
+            or up.dtype != gate.dtype or up.shape[0] != gate.shape[0]:
+        raise ValueError("glu_act: gate and up are [n, >= ff] of one dtype with unit inner strides")
+    out = torch.empty(gate.shape[0], ff, dtype=gate.dtype, device=gate.device)
+    L.check(L.lib().ll_glu_act(out.data_ptr(), gate.data_ptr(), gate.stride(0), up.data_ptr(), up.stride(0), gate.shape[0], int(ff),
+                               _GLU_KINDS[kind], L.dtype_code(gate.dtype), L.stream_ptr()), "glu_act")
+    return out
+
+
+@torch.no_grad()
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` in place (fp32 arithmetic)."""
+    L.require_cuda(x)
+    if not x.is_contiguous():
+        raise ValueError("softcap_: a contiguous tensor")
+    L.check(L.lib().ll_softcap(x.data_ptr(), x.numel(), float(cap), L.dtype_code(x.dtype), L.stream_ptr()), "softcap")
+    return x

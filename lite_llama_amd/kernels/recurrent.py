@@ -47,3 +47,28 @@ def gated_linear_scan(qfv: torch.Tensor, heads: int, dk: int, dv: int, f_bias, l
         L.dtype_code(dt), L.stream_ptr()),
         "gated_linear_scan")
     return out
+
+
+@torch.no_grad()
+def mingru_scan(zxg: torch.Tensor, width: int, z_bias, x_bias, step, state: torch.Tensor) -> torch.Tensor:
+    """minGRU over a ragged step.  ``zxg [n, >= 3 width]`` = fused projection rows ``[z_raw | x_raw | g_raw]``; per channel
+    ``z = sigmoid(z_raw + z_bias)``, ``u = x_raw + x_bias``, candidate ``u + 1/2`` where ``u >= 0`` and ``sigmoid(u)`` below,
+    ``S <- (1 - z) S + z candidate``; returns ``S * silu(g_raw)`` ``[n, width]`` in the storage dtype.  ``state
+    [slots, width]`` fp32: a sequence whose run starts at position 0 starts from zeros, every run leaves its final state."""
+    L.require_cuda(zxg, z_bias, x_bias, state)
+    n, dt = zxg.shape[0], zxg.dtype
+    if zxg.dim() != 2 or zxg.stride(1) != 1 or zxg.shape[1] < 3 * width:
+        raise ValueError("mingru_scan: rows hold [z | x | g]")
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 2 or state.shape[1] != width:
+        raise ValueError("mingru_scan: state is contiguous fp32 [slots, width]")
+    for b in (z_bias, x_bias):
+        if b is not None and (b.dtype != dt or b.numel() != width or not b.is_contiguous()):
+            raise ValueError("mingru_scan: biases are [width] in the rows' dtype")
+    if step.num_tokens != n:
+        raise ValueError("mingru_scan: the step describes another number of tokens")
+    out = torch.empty(n, width, dtype=dt, device=zxg.device)
+    es, base = zxg.element_size(), zxg.data_ptr()
+    L.check(L.lib().ll_mingru_scan(base, base + width * es, base + 2 * width * es, zxg.stride(0), L.ptr(z_bias), L.ptr(x_bias),
+                                   out.data_ptr(), step.num_seqs, width, step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(),
+                                   step.seq_slot.data_ptr(), state.data_ptr(), L.dtype_code(dt), L.stream_ptr()), "mingru_scan")
+    return out

@@ -9,15 +9,25 @@ description, out of mixers that take a ragged step (executor/ragged.py) and keep
   * :class:`GatedLinearMixer`  HGRN2: linear attention whose forget gate, bounded from below, also decides what is written
                                (kernels/recurrent.py)
   * :class:`DenseMLP`          ``down(act(up h))`` with the xIELU activation (kernels/activations.py)
+  * :class:`LatentAttention`   attention over a shared low-rank latent with a rotated key part common to all heads, run in the
+                               absorbed form (one key/value head over the cached latent rows), optionally with a query latent,
+                               a sliding window and an output gate (kernels/attention.py)
+  * :class:`MinGRU`            a per-channel gated recurrence whose gates read the current token only (kernels/recurrent.py)
+  * :class:`GatedMLP`          ``down(act(gate h) * up h)`` (silu or tanh-gelu)
+  * :class:`SparseMoE`         sigmoid router over expert groups, grouped expert products, a shared expert with a per-token
+                               scale (kernels/fused_moe.py)
 
 The residual stream is fp32 throughout; every layer's residual add is fused into the norm that follows it
-(kernels/norm_act.py::add_rmsnorm_shift), which also applies the token shift in front of a mixer.  Projections run through the
-framework's linear layers (library GEMM for unquantised weights), with q|f|v and q|k|v fused into one launch at load time.
-The first family built this way is Rakevik (``"architecture": "Rakevik"``).
+(kernels/norm_act.py::add_rmsnorm_shift, which also applies the token shift in front of a mixer; or
+kernels/norm_act.py::gated_group_norm for layers that wrap each sublayer in two grouped norms and gate its result).
+Projections run through the framework's linear layers (library GEMM for unquantised weights), with everything that reads one
+input fused into one launch at load time.  Families: Rakevik (``"architecture": "Rakevik"``: :class:`MixerLayer`) and
+Rukedra (:class:`SandwichLayer`).
 """
 
 from __future__ import annotations
 
+import math
 from collections.abc import Mapping
 from dataclasses import dataclass, field
 
@@ -27,9 +37,10 @@ import torch.nn.functional as F
 
 from .distributed.parallel_state import get_tp_world_size
 from .kernels.activations import xielu
-from .kernels.attention import qk_norm_cache, ragged_attention
-from .kernels.norm_act import add_rmsnorm_shift, cast_pair, residual_set
-from .kernels.recurrent import gated_linear_scan
+from .kernels.attention import latent_kv_prep, qk_norm_cache, ragged_attention, rotate_pairs
+from .kernels.fused_moe import group_router, sparse_glu_experts
+from .kernels.norm_act import GatedUpdate, add_rmsnorm_shift, cast_pair, gated_group_norm, glu_act, residual_set, softcap_
+from .kernels.recurrent import gated_linear_scan, mingru_scan
 from .linear import ReplicatedLinear
 
 
@@ -37,15 +48,71 @@ from .linear import ReplicatedLinear
 # description
 # ------------------------------------------------------------------------------------- #
 @dataclass(frozen=True)
+class RotarySpec:
+    """Rotation of entry pairs (2i, 2i + 1) of the first ``dims`` entries by ``position * f_i``, ``f_i = base^(-2i / dims)``;
+    with ``factor`` the frequencies are rescaled between a fast and a slow end (YaRN)."""
+    dims: int
+    base: float
+    factor: float = 0.0         # 0: no scaling
+    original: float = 0.0       # positions the unscaled frequencies were made for
+    fast: float = 32.0          # turns over `original` positions above which a pair keeps its frequency
+    slow: float = 1.0           # ... and below which it is divided by `factor`
+
+    def table(self) -> tuple[list[float], float]:
+        """``(frequency per pair, amplitude of cos / sin)``."""
+        half = self.dims // 2
+        f = [self.base ** (-2.0 * i / self.dims) for i in range(half)]
+        if not self.factor:
+            return f, 1.0
+
+        def pair_of(turns: float) -> float:   # the (fractional) pair that makes `turns` turns over `original` positions
+            return self.dims * math.log(self.original / (2 * math.pi * turns)) / (2 * math.log(self.base))
+
+        lo = max(math.floor(pair_of(self.fast)), 0)
+        hi = min(math.ceil(pair_of(self.slow)), self.dims - 1)
+        out = []
+        for i, fi in enumerate(f):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            out.append(fi / self.factor * ramp + fi * (1.0 - ramp))
+        return out, 0.1 * math.log(self.factor) + 1.0
+
+    @staticmethod
+    def from_config(rot: Mapping) -> "RotarySpec":
+        sc = rot.get("scaling") or {}
+        return RotarySpec(int(rot["dims"]), float(rot["base"]), float(sc.get("factor", 0.0)), float(sc.get("original", 0.0)),
+                          float(sc.get("fast", 32.0)), float(sc.get("slow", 1.0)))
+
+
+@dataclass(frozen=True)
 class MixerSpec:
-    kind: str                   # "attention" | "hgrn2"
-    heads: int
-    dim: int                    # per-head query / key width
-    vdim: int                   # per-head value width
+    kind: str                   # "attention" | "hgrn2" | "latent_attention" | "mingru"
+    heads: int = 1
+    dim: int = 0                # per-head query / key width (latent attention: the unrotated part)
+    vdim: int = 0               # per-head value width
     kv_heads: int = 0           # attention only
-    scale: float = 1.0          # attention only
+    scale: float = 1.0          # attention kinds
     temp_coef: float = 0.0      # attention only: q *= 1 + temp_coef ln(floor((p + 1) / temp_every) + 1)
     temp_every: int = 1
+    rot_dim: int = 0            # latent attention: rotated query / key entries per head (the key's are shared by all heads)
+    kv_rank: int = 0            # latent attention: width of the cached key/value latent
+    q_rank: int = 0             # latent attention: width of the query latent (0: queries are projected directly)
+    window: int = 0             # latent attention: 0 = causal, else the last `window` positions are seen
+    out_gate: bool = False      # latent attention: heads times sigmoid(W_g h) before the output projection
+    rotary: RotarySpec | None = None
+    width: int = 0              # mingru: channels of the recurrence
+
+
+@dataclass(frozen=True)
+class MlpSpec:
+    kind: str = "dense"         # "dense" | "moe"
+    ff: int = 0                 # dense: hidden width; moe: hidden width of one expert
+    act: str = "xielu"          # dense: "xielu" (up / down) | "gelu_tanh" (gate / up / down)
+    experts: int = 0
+    top: int = 0
+    group_count: int = 1
+    group_keep: int = 1
+    route_scale: float = 1.0
+    shared_ff: int = 0          # 0: no shared expert
 
 
 @dataclass(frozen=True)
@@ -53,6 +120,8 @@ class LayerSpec:
     mixer: MixerSpec
     ff: int = 0                 # 0: the layer has no feed-forward sublayer
     mlp_kind: str = "dense"
+    mlp: MlpSpec | None = None
+    weights_of: int | None = None   # the layer whose parameters this one uses (its cache / state stays its own)
 
 
 @dataclass(frozen=True)
@@ -66,6 +135,9 @@ class LayeredGeometry:
     loop_stop: int = 0
     loop_times: int = 1
     token_shift: bool = True
+    sandwich: bool = False      # every sublayer between two norms, its result gated by sigmoid(W_r h + b_r)
+    norm_groups: int = 1        # norms are taken over this many equal consecutive parts of the row
+    logit_softcap: float = 0.0  # logits <- cap tanh(logits / cap)
     extra: dict = field(default_factory=dict, compare=False)
 
     @property
@@ -84,6 +156,8 @@ class LayeredGeometry:
 
     @staticmethod
     def from_config(config: Mapping, name: str = "rakevik") -> "LayeredGeometry":
+        if name == "rukedra":
+            return _rukedra_geometry(config, name)
         layers = []
         for entry in config["layers"]:
             m, kind = entry["mixer"], entry["type"]
@@ -109,6 +183,55 @@ class LayeredGeometry:
         return LayeredGeometry(name=name, vocab_size=int(config["vocab"]), width=int(config["width"]),
                                eps=float(config["norm"]["eps"]), layers=tuple(layers), loop_start=start, loop_stop=stop,
                                loop_times=times if stop > start else 1)
+
+
+def _rukedra_geometry(config: Mapping, name: str) -> LayeredGeometry:
+    """Rukedra: latent attention (two variants) and minGRU mixers, dense (tanh-gelu) and mixture-of-experts feed-forwards,
+    grouped norms before and after every sublayer, gated residual branches, layers that borrow another layer's weights."""
+    layers = []
+    for index, entry in enumerate(config["layers"]):
+        m, kind = entry["mixer"], entry["type"]
+        if kind in ("latent_attention", "latent_attention_2"):
+            first = kind == "latent_attention"
+            rot = RotarySpec.from_config(m["rot"])
+            spec = MixerSpec("latent_attention", heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                             scale=float(m["scale"]), rot_dim=int(m["rot_dim"]), kv_rank=int(m["kv_rank"]),
+                             q_rank=int(m["q_rank"]) if first else 0, window=int((m.get("mask") or {}).get("size", 0)) if first else 0,
+                             out_gate=first, rotary=rot)
+            if rot.dims > spec.rot_dim or rot.dims % 2:
+                raise ValueError(f"layer {index}: {rot.dims} rotated entries do not fit a rotated part of {spec.rot_dim}")
+        elif kind == "mingru":
+            spec = MixerSpec("mingru", width=int(m["width"]))
+        else:
+            raise ValueError(f"unsupported mixer type {kind!r}; supported: latent_attention, latent_attention_2, mingru")
+        mlp = entry.get("mlp")
+        if mlp is None:
+            mspec = None
+        elif mlp.get("kind", "dense") == "dense":
+            mspec = MlpSpec("dense", ff=int(mlp["ff"]), act="gelu_tanh")
+        elif mlp["kind"] == "moe":
+            r = mlp["router"]
+            groups = r.get("groups") or {}
+            mspec = MlpSpec("moe", ff=int(mlp["expert"]["ff"]), act="silu", experts=int(r["experts"]), top=int(r["top"]),
+                            group_count=int(groups.get("count", 1)), group_keep=int(groups.get("keep", 1)),
+                            route_scale=float(r.get("scale", 1.0)), shared_ff=int((mlp.get("shared") or {}).get("ff", 0)))
+            if mspec.experts % mspec.group_count or mspec.group_keep * (mspec.experts // mspec.group_count) < mspec.top:
+                raise ValueError(f"layer {index}: {mspec.top} of {mspec.experts} experts cannot be chosen from "
+                                 f"{mspec.group_keep} of {mspec.group_count} groups")
+        else:
+            raise ValueError(f"unsupported feed-forward kind {mlp.get('kind')!r}; supported: dense, moe")
+        owner = entry.get("weights_of")
+        if owner is not None and not (0 <= int(owner) < index and config["layers"][int(owner)].get("weights_of") is None):
+            raise ValueError(f"layer {index} borrows the weights of layer {owner}, which is not an earlier layer with its own")
+        layers.append(LayerSpec(spec, ff=mspec.ff if mspec else 0, mlp_kind=mspec.kind if mspec else "dense", mlp=mspec,
+                                weights_of=None if owner is None else int(owner)))
+    norm = config["norm"]
+    groups = int(norm.get("groups", 1))
+    if int(config["width"]) % groups:
+        raise ValueError(f"{groups} norm groups do not divide the width {config['width']}")
+    return LayeredGeometry(name=name, vocab_size=int(config["vocab"]), width=int(config["width"]), eps=float(norm["eps"]),
+                           layers=tuple(layers), token_shift=False, sandwich=True, norm_groups=groups,
+                           logit_softcap=float(config.get("logit_softcap") or 0.0))
 
 
 def _linear(inp: int, out: int) -> ReplicatedLinear:
@@ -183,7 +306,128 @@ class DenseMLP(nn.Module):
         return self.down_proj(xielu(self.up_proj(h), self.act))
 
 
-MIXERS = {"attention": SinkAttention, "hgrn2": GatedLinearMixer}
+class LatentAttention(nn.Module):
+    """Attention whose keys and values are up-projections of ONE cached latent row per token, plus a rotated key part that
+    all heads share.  Run in the absorbed form: the cache holds ``[latent | rotated key part]`` (one key/value head of key
+    width ``kv_rank + rot_dim``; the values are the first ``kv_rank`` columns of the same rows), a head's query becomes
+    ``[W_uk^T q_unrotated | rotate(q_rotated)]`` and its output ``W_uv (weights . latents)`` -- two batched products over the
+    heads around the attention kernel.  Everything that reads the mixer's input (query or query latent, key/value latent,
+    output gate, ``extra`` columns of the layer) is one projection."""
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float, extra: int = 0):
+        super().__init__()
+        self.spec, self.eps, self.extra = spec, eps, extra
+        s = spec
+        self.q_width = s.heads * (s.dim + s.rot_dim)
+        q_cols = s.q_rank if s.q_rank else self.q_width
+        self.kv_off = q_cols
+        self.gate_off = q_cols + s.kv_rank + s.rot_dim
+        self.extra_off = self.gate_off + (s.heads * s.vdim if s.out_gate else 0)
+        self.in_proj = _linear(width, self.extra_off + extra)
+        if s.q_rank:
+            self.q_norm_weight = _vector(s.q_rank)
+            self.uq_proj = _linear(s.q_rank, self.q_width)
+        self.kv_norm_weight = _vector(s.kv_rank)
+        self.uk_weight = nn.Parameter(torch.zeros(s.heads * s.dim, s.kv_rank, dtype=torch.float16), requires_grad=False)
+        self.uv_weight = nn.Parameter(torch.zeros(s.heads * s.vdim, s.kv_rank, dtype=torch.float16), requires_grad=False)
+        self.o_proj = _linear(s.heads * s.vdim, width)
+        self._freq_values, self.amp = s.rotary.table()
+        self.pairs = len(self._freq_values)
+        self._freq = None   # fp32 on the device of the first step (not a buffer: a module-wide cast must not touch the angles)
+
+    def cache_run(self) -> dict:
+        return {"kind": "latent", "rank": self.spec.kv_rank, "rot": self.spec.rot_dim}
+
+    def forward(self, h, step, cache, run: int, token_table):
+        s = self.spec
+        n = h.shape[0]
+        rows = self.in_proj(h)
+        k_cache, v_cache = cache.kv_buffer[run]
+        if self._freq is None or self._freq.device != h.device:
+            self._freq = torch.tensor(self._freq_values, dtype=torch.float64).to(torch.float32).to(h.device)
+        c_q = latent_kv_prep(rows, self.kv_off, s.kv_rank, s.rot_dim, self.kv_norm_weight, self.eps, self._freq, self.pairs, self.amp,
+                             step, k_cache.view(k_cache.shape[0], -1), q_off=0, q_rank=s.q_rank,
+                             q_norm_weight=self.q_norm_weight if s.q_rank else None)
+        q = (self.uq_proj(c_q) if s.q_rank else rows[:, :self.q_width]).view(n, s.heads, s.dim + s.rot_dim)
+        qa = torch.empty(n, s.heads, s.kv_rank + s.rot_dim, dtype=h.dtype, device=h.device)
+        # absorbed query: [heads, n, dim] x [heads, dim, rank] straight into the front columns of the query rows
+        torch.bmm(q[:, :, :s.dim].transpose(0, 1), self.uk_weight.view(s.heads, s.dim, s.kv_rank),
+                  out=qa[:, :, :s.kv_rank].transpose(0, 1))
+        rotate_pairs(q, s.dim, s.rot_dim, self._freq, self.pairs, self.amp, step, qa, s.kv_rank)
+        o_lat = ragged_attention(qa, k_cache, v_cache, s.scale, step, token_table, window=s.window)     # [n, heads * rank]
+        o = torch.empty(n, s.heads, s.vdim, dtype=h.dtype, device=h.device)
+        torch.bmm(o_lat.view(n, s.heads, s.kv_rank).transpose(0, 1), self.uv_weight.view(s.heads, s.vdim, s.kv_rank).transpose(1, 2),
+                  out=o.transpose(0, 1))
+        o = o.view(n, s.heads * s.vdim)
+        if s.out_gate:
+            o = glu_act(rows[:, self.gate_off:], s.heads * s.vdim, "sigmoid", up=o)
+        return self.o_proj(o), (rows[:, self.extra_off:] if self.extra else None)
+
+
+class MinGRU(nn.Module):
+    """``z | x | g`` (and ``extra`` columns of the layer) in one projection; gates, recurrence and the silu-gated read-out in
+    one launch over the fp32 state slots; output projection."""
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float, extra: int = 0):
+        super().__init__()
+        self.spec, self.extra = spec, extra
+        self.in_proj = _linear(width, 3 * spec.width + extra)
+        self.z_bias = _vector(spec.width)
+        self.x_bias = _vector(spec.width)
+        self.o_proj = _linear(spec.width, width)
+
+    def cache_run(self) -> dict:
+        return {"kind": "recurrent", "heads": 1, "dk": 1, "dv": self.spec.width}
+
+    def forward(self, h, step, cache, run: int, token_table):
+        w = self.spec.width
+        rows = self.in_proj(h)
+        o = mingru_scan(rows, w, self.z_bias, self.x_bias, step, cache.recurrent[run].view(-1, w))
+        return self.o_proj(o), (rows[:, 3 * w:] if self.extra else None)
+
+
+class GatedMLP(nn.Module):
+    """``down(act(gate h) * (up h))``; ``gate | up`` (and ``extra`` columns of the layer) are one projection."""
+
+    def __init__(self, width: int, ff: int, act: str, extra: int = 0):
+        super().__init__()
+        self.ff, self.act, self.extra = ff, act, extra
+        self.in_proj = _linear(width, 2 * ff + extra)
+        self.down_proj = _linear(ff, width)
+
+    def forward(self, h):
+        rows = self.in_proj(h)
+        return self.down_proj(glu_act(rows, self.ff, self.act)), (rows[:, 2 * self.ff:] if self.extra else None), None, None
+
+
+class SparseMoE(nn.Module):
+    """Sigmoid router over expert groups (fp32), the chosen experts' gated feed-forwards as grouped products over slots sorted
+    by expert, and a shared expert whose result is scaled per token by ``sigmoid(w_sg . h)``.  The slots' rows are NOT summed
+    here: they ride, with the shared row and its scale, into the norm launch that follows."""
+
+    def __init__(self, width: int, spec: MlpSpec, extra: int = 0):
+        super().__init__()
+        self.spec, self.extra = spec, extra
+        self.router_weight = nn.Parameter(torch.zeros(spec.experts, width, dtype=torch.float16), requires_grad=False)
+        self.gate_up_weight = nn.Parameter(torch.zeros(spec.experts, 2 * spec.ff, width, dtype=torch.float16), requires_grad=False)
+        self.down_weight = nn.Parameter(torch.zeros(spec.experts, width, spec.ff, dtype=torch.float16), requires_grad=False)
+        if spec.shared_ff or extra:
+            self.in_proj = _linear(width, 2 * spec.shared_ff + extra)   # shared gate | shared up | the layer's columns
+        if spec.shared_ff:
+            self.shared_down_proj = _linear(spec.shared_ff, width)
+            self.shared_scale_weight = nn.Parameter(torch.zeros(1, width, dtype=torch.float16), requires_grad=False)
+
+    def forward(self, h):
+        s = self.spec
+        ids, weights, scale = group_router(h, self.router_weight, s.top, s.group_count, s.group_keep, s.route_scale,
+                                           extra_weight=self.shared_scale_weight if s.shared_ff else None)
+        y = sparse_glu_experts(h, self.gate_up_weight, self.down_weight, ids, weights)
+        rows = self.in_proj(h) if (s.shared_ff or self.extra) else None
+        shared = self.shared_down_proj(glu_act(rows, s.shared_ff, "silu")) if s.shared_ff else None
+        return y, (rows[:, 2 * s.shared_ff:] if self.extra else None), shared, scale
+
+
+MIXERS = {"attention": SinkAttention, "hgrn2": GatedLinearMixer, "latent_attention": LatentAttention, "mingru": MinGRU}
 
 
 class MixerLayer(nn.Module):
@@ -206,6 +450,37 @@ class MixerLayer(nn.Module):
         return x, delta
 
 
+class SandwichLayer(nn.Module):
+    """``x <- x + norm_b(f(norm_a(x)) * sigmoid(W_r norm_a(x) + b_r))`` for the mixer and then for the feed-forward, norms
+    over groups.  ``W_r`` rides as extra columns in the sublayer's input projection; a sublayer's result is carried as a
+    :class:`GatedUpdate` into the norm launch that opens the next sublayer (gate, post-norm, residual add and pre-norm are one
+    launch)."""
+
+    def __init__(self, geo: LayeredGeometry, spec: LayerSpec):
+        super().__init__()
+        self.eps, self.groups = geo.eps, geo.norm_groups
+        w = geo.width
+        self.norm1_weight, self.norm1b_weight = _vector(w), _vector(w)
+        self.rg1_bias = _vector(w)
+        self.mixer = MIXERS[spec.mixer.kind](w, spec.mixer, geo.eps, extra=w)
+        self.mlp = None
+        if spec.mlp is not None:
+            self.norm2_weight, self.norm2b_weight = _vector(w), _vector(w)
+            self.rg2_bias = _vector(w)
+            self.mlp = SparseMoE(w, spec.mlp, extra=w) if spec.mlp.kind == "moe" else GatedMLP(w, spec.mlp.ff, spec.mlp.act, extra=w)
+
+    def forward(self, x, pending, step, cache, run: int, token_table):
+        """``(x, pending)``: the fp32 residual (updated in place) and the update still to enter it.  Returns the same pair."""
+        h = gated_group_norm(x, pending, self.norm1_weight, self.eps, self.groups)
+        y, gate = self.mixer(h, step, cache, run, token_table)
+        pending = GatedUpdate(y, self.norm1b_weight, gate, self.rg1_bias)
+        if self.mlp is not None:
+            h = gated_group_norm(x, pending, self.norm2_weight, self.eps, self.groups)
+            y, gate, shared, scale = self.mlp(h)
+            pending = GatedUpdate(y, self.norm2b_weight, gate, self.rg2_bias, shared, scale)
+        return x, pending
+
+
 # ------------------------------------------------------------------------------------- #
 # the model
 # ------------------------------------------------------------------------------------- #
@@ -219,7 +494,11 @@ class LayeredLM(nn.Module):
         self.geo = geo
         self.embed_tokens = nn.Embedding(geo.vocab_size, geo.width, dtype=torch.float16)
         self.embed_tokens.weight.requires_grad_(False)
-        self.layers = nn.ModuleList(MixerLayer(geo, spec) for spec in geo.layers)
+        make = SandwichLayer if geo.sandwich else MixerLayer
+        built: list[nn.Module] = []
+        for spec in geo.layers:   # a layer that borrows weights IS the other layer's module; its cache run stays its own
+            built.append(built[spec.weights_of] if spec.weights_of is not None else make(geo, spec))
+        self.layers = nn.ModuleList(built)
         if geo.looped:
             self.loop_in = _linear(2 * geo.width, geo.width)
             self.loop_step = nn.Parameter(torch.zeros(geo.loop_times, geo.width, dtype=torch.float16), requires_grad=False)
@@ -238,7 +517,7 @@ class LayeredLM(nn.Module):
         for index, _, _ in self.run_order:
             layer = self.layers[index]
             run = layer.mixer.cache_run()
-            if layer.shift is not None:
+            if getattr(layer, "shift", None) is not None:
                 run["shift_width"] = self.geo.width
             runs.append(run)
         return runs
@@ -256,13 +535,23 @@ class LayeredLM(nn.Module):
                 x, delta = residual_set(y, self.loop_step[pass_no]), None
             x, delta = self.layers[index](x, delta, step, cache, run, token_table)
             if collect_layers is not None:
-                collect_layers.append(x + delta.float() if delta is not None else x.clone())
+                if self.geo.sandwich:   # (diagnostics: the pending update is applied to a copy)
+                    seen = x.clone()
+                    gated_group_norm(seen, delta, None, self.geo.eps, self.geo.norm_groups)
+                    collect_layers.append(seen)
+                else:
+                    collect_layers.append(x + delta.float() if delta is not None else x.clone())
         if logits_rows is None:
             return None
         x = x[logits_rows].contiguous()
-        delta = delta[logits_rows].contiguous() if delta is not None else None
-        h, _ = add_rmsnorm_shift(x, delta, self.norm_weight, self.geo.eps, x_out=x)
-        return self.lm_head(h)
+        if self.geo.sandwich:
+            h = gated_group_norm(x, delta.rows(logits_rows) if delta is not None else None, self.norm_weight, self.geo.eps,
+                                 self.geo.norm_groups)
+        else:
+            delta = delta[logits_rows].contiguous() if delta is not None else None
+            h, _ = add_rmsnorm_shift(x, delta, self.norm_weight, self.geo.eps, x_out=x)
+        logits = self.lm_head(h)
+        return softcap_(logits, self.geo.logit_softcap) if self.geo.logit_softcap else logits
 
     # --------------------------------------------------------------------------------- #
     # synthetic weights (benchmarks, tests): seeded, every tensor in a range that keeps the stack well-conditioned

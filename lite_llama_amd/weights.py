@@ -577,17 +577,84 @@ def _layered_translator(geo) -> Translator:
     return translate
 
 
+def _rukedra_translator(geo) -> Translator:
+    """Tensor names of a Rukedra checkpoint -> parameters of :class:`lite_llama_amd.model_layers.LayeredLM` built from
+    :class:`SandwichLayer`: everything that reads a sublayer's input (``mix.dq`` / ``mix.q``, ``mix.dkv``, ``mix.g``,
+    ``mix.z``, ``mix.x``, the residual gate ``rg1``; ``mlp.gate``, ``mlp.up``, ``mlp.shared.gate``, ``mlp.shared.up``, ``rg2``)
+    lands in its row range of that sublayer's one input projection; experts ``mlp.e<k>.*`` land in the stacked expert
+    tensors.  A layer that borrows another layer's weights has no tensors of its own."""
+    fixed = {"embed": "embed_tokens.weight", "final.norm": "norm_weight", "head": "lm_head.weight"}
+    plain = {"norm1": "norm1_weight", "norm1b": "norm1b_weight", "norm2": "norm2_weight", "norm2b": "norm2b_weight",
+             "rg1.b": "rg1_bias", "rg2.b": "rg2_bias", "mix.o": "mixer.o_proj.weight", "mix.dq.norm": "mixer.q_norm_weight",
+             "mix.uq": "mixer.uq_proj.weight", "mix.dkv.norm": "mixer.kv_norm_weight", "mix.uk": "mixer.uk_weight",
+             "mix.uv": "mixer.uv_weight", "mix.z.b": "mixer.z_bias", "mix.x.b": "mixer.x_bias", "mlp.down": "mlp.down_proj.weight",
+             "mlp.router": "mlp.router_weight", "mlp.shared.down": "mlp.shared_down_proj.weight",
+             "mlp.shared.sg": "mlp.shared_scale_weight"}
+    expert_leaf = re.compile(r"^mlp\.e(\d+)\.(gate|up|down)$")
+
+    def fused(spec):
+        """``{checkpoint leaf: (parameter, first row, rows)}`` of the layer's two input projections."""
+        m, w, out = spec.mixer, geo.width, {}
+        if m.kind == "latent_attention":
+            q_width = m.heads * (m.dim + m.rot_dim)
+            q_cols = m.q_rank or q_width
+            out["mix.dq" if m.q_rank else "mix.q"] = ("mixer.in_proj.weight", 0, q_cols)
+            out["mix.dkv"] = ("mixer.in_proj.weight", q_cols, m.kv_rank + m.rot_dim)
+            at = q_cols + m.kv_rank + m.rot_dim
+            if m.out_gate:
+                out["mix.g"] = ("mixer.in_proj.weight", at, m.heads * m.vdim)
+                at += m.heads * m.vdim
+            out["rg1"] = ("mixer.in_proj.weight", at, w)
+        else:
+            for k, leaf in enumerate(("mix.z", "mix.x", "mix.g")):
+                out[leaf] = ("mixer.in_proj.weight", k * m.width, m.width)
+            out["rg1"] = ("mixer.in_proj.weight", 3 * m.width, w)
+        mlp = spec.mlp
+        if mlp is not None and mlp.kind == "dense":
+            out["mlp.gate"], out["mlp.up"] = ("mlp.in_proj.weight", 0, mlp.ff), ("mlp.in_proj.weight", mlp.ff, mlp.ff)
+            out["rg2"] = ("mlp.in_proj.weight", 2 * mlp.ff, w)
+        elif mlp is not None:
+            if mlp.shared_ff:
+                out["mlp.shared.gate"] = ("mlp.in_proj.weight", 0, mlp.shared_ff)
+                out["mlp.shared.up"] = ("mlp.in_proj.weight", mlp.shared_ff, mlp.shared_ff)
+            out["rg2"] = ("mlp.in_proj.weight", 2 * mlp.shared_ff, w)
+        return out
+
+    members = [fused(spec) if spec.weights_of is None else {} for spec in geo.layers]
+
+    def translate(key: str) -> Target:
+        if key in fixed:
+            return fixed[key], whole
+        m = re.match(r"^l(\d+)\.(.+)$", key)
+        if m is None or int(m.group(1)) >= len(geo.layers):
+            return key, whole  # unknown: load_weights reports it
+        index, leaf = int(m.group(1)), m.group(2)
+        if leaf in members[index]:
+            name, first, rows = members[index][leaf]
+            return f"layers.{index}.{name}", Region(rows=(first, rows))
+        e = expert_leaf.match(leaf)
+        if e is not None:
+            k, proj = int(e.group(1)), e.group(2)
+            if proj == "down":
+                return f"layers.{index}.mlp.down_weight", expert(k)
+            return f"layers.{index}.mlp.gate_up_weight", expert_half(k, 0 if proj == "gate" else 1)
+        return f"layers.{index}.{plain.get(leaf, leaf)}", whole
+
+    return translate
+
+
 def _load_layered(config: Mapping, checkpoints_dir, device, dtype=None, **_):
     from .model_layers import LayeredGeometry, LayeredLM
 
     geo = LayeredGeometry.from_config(config, name=model_family(config))
     model = LayeredLM(geo, dtype=dtype or torch.bfloat16).to(device)
+    translator = _rukedra_translator(geo) if geo.sandwich else _layered_translator(geo)
     with torch.no_grad():
-        load_weights(model, hf_weights_iterator(checkpoints_dir, device), _layered_translator(geo))
+        load_weights(model, hf_weights_iterator(checkpoints_dir, device), translator)
     return model.eval()
 
 
-MODEL_FAMILIES: dict[str, Callable] = {"rakevik": _load_layered}
+MODEL_FAMILIES: dict[str, Callable] = {"rakevik": _load_layered, "rukedra": _load_layered}
 
 
 def load_pretrained(checkpoints_dir: str | Path, *, device: str | torch.device = "cuda", quantization: str | None = None,
