@@ -61,12 +61,14 @@ def yarn_frequencies(rot):
     return torch.tensor(out, dtype=torch.float64), 0.1 * math.log(factor) + 1.0
 
 
-def rotate_pairs(v, positions, rot):
+def rotate_pairs(v, positions, rot, angle_dtype=torch.float64):
     """``v [T, ..., n]``: the first ``rot.dims`` entries of the last axis are rotated pair by pair -- entry 2i with entry
-    2i + 1 -- by the angle ``position * f_i``; cos and sin carry the amplitude.  The rest passes unchanged."""
+    2i + 1 -- by the angle ``position * f_i``; cos and sin carry the amplitude.  The rest passes unchanged.  ``angle_dtype``:
+    the precision in which frequency and angle are held (the design computes them in 32 bits: far out, that rounding of the
+    angle is larger than anything else in the rotation)."""
     f, amp = yarn_frequencies(rot)
     dims = int(rot["dims"])
-    ang = positions.to(torch.float64)[:, None] * f[None, :]
+    ang = (positions.to(angle_dtype)[:, None] * f.to(angle_dtype)[None, :]).to(torch.float64)
     cos, sin = (torch.cos(ang) * amp).to(v.dtype), (torch.sin(ang) * amp).to(v.dtype)
     while cos.dim() < v.dim():
         cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
