@@ -95,6 +95,12 @@ def parse():
                     help="instead of the headline: prefill / decode throughput and per-kernel roofline fractions of the layered "
                          "family (model_layers.py) beside the closest llama-shaped model at equal sizes (benchmarks/layered_bench.py)")
     ap.add_argument("--layered-dtype", default="bf16", choices=["bf16", "f16", "f32"])
+    ap.add_argument("--rukedra", action="store_true",
+                    help="instead of the headline: prefill / decode throughput and per-kernel roofline fractions of the Rukedra "
+                         "design (latent attention, minGRU, gated grouped norms, routed experts) at two model sizes beside the "
+                         "closest llama-shaped model (benchmarks/rukedra_bench.py); --layered-dtype picks the dtype")
+    ap.add_argument("--rukedra-sizes", default="compact,wide", help="which size points of benchmarks/rukedra_bench.py::SIZES to run")
+    ap.add_argument("--rukedra-model-only", action="store_true", help="skip the per-kernel table (a short run for a kernel trace)")
     ap.add_argument("--no-reference-order", action="store_true",
                     help="skip the bounded drop-in-route entry (\"reference_order\") of the default N = 1 int4 line")
     return ap.parse_args()
@@ -923,6 +929,11 @@ def main():
         from benchmarks.layered_bench import run as layered_run
 
         print(json.dumps(layered_run(args.layered_dtype)))
+        return
+    if args.rukedra:
+        from benchmarks.rukedra_bench import run as rukedra_run
+
+        print(json.dumps(rukedra_run(args.layered_dtype, sizes=tuple(args.rukedra_sizes.split(",")), kernels=not args.rukedra_model_only)))
         return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         raise SystemExit(self_launch(args))

@@ -655,20 +655,21 @@ int ll_rotate_pairs(const void* q, int64_t q_tok_stride, int64_t q_head_stride, 
  * ll_group_router: scores = sigmoid(W_router h) in fp32; experts in group_count equal groups of neighbours, group score = sum
  * of its two best, the best group_keep groups stay eligible; ids [n, top] / weights [n, top] (fp32) = the top eligible experts
  * by score and score / (sum + 1e-20) * route_scale.  w_extra [width] (or NULL): extra_scale[t] = sigmoid(w_extra . h).
- * ll_moe_sort: slots sorted by expert in blocks of ll_moe_rows_block() rows (counts: int32 scratch [experts]; sorted
- * [num_slots + experts (block - 1)], block_expert [ceil(that / block)], num_post [1]).
+ * logits: fp32 scratch [n][experts + (w_extra ? 1 : 0)].
+ * ll_moe_sort: slots sorted by expert in blocks of `block` = ll_moe_rows_block(...) rows, 32 or 128 (counts: int32 scratch
+ * [experts]; sorted [num_slots + experts (block - 1)], block_expert [ceil(that / block)], num_post [1]).
  * ll_moe_rows_gemm: glu != 0: w [experts][2 N][K] (gate rows, then up rows), out[slot] = silu(a Wg^T) * (a Wu^T) with
  * a = row slot / a_div; glu == 0: w [experts][N][K], out[slot] = (a W^T) * slot_weight[slot]. */
 int ll_group_router(const void* h, int64_t h_ld, const void* w_router, const void* w_extra, int64_t n, int64_t width,
                     int64_t experts, int64_t top, int64_t group_count, int64_t group_keep, float route_scale,
-                    int32_t* ids, float* weights, float* extra_scale, int dtype, void* stream);
-int64_t ll_moe_rows_block(void);
-int ll_moe_sort(const int32_t* ids, int64_t num_slots, int64_t experts, int32_t* counts, int32_t* sorted,
+                    int32_t* ids, float* weights, float* extra_scale, float* logits, int dtype, void* stream);
+int64_t ll_moe_rows_block(int64_t num_slots, int64_t experts, int64_t width, int64_t ff, int dtype);
+int ll_moe_sort(const int32_t* ids, int64_t num_slots, int64_t experts, int64_t block, int32_t* counts, int32_t* sorted,
                 int32_t* block_expert, int32_t* num_post, void* stream);
 int ll_moe_rows_gemm(const void* a, int64_t a_ld, int64_t a_div, const void* w, int64_t w_stride_e, int64_t K, int64_t N,
                      int glu, const float* slot_weight, void* out, int64_t out_ld, const int32_t* sorted,
-                     const int32_t* block_expert, const int32_t* num_post, int64_t num_slots, int64_t experts, int dtype,
-                     void* stream);
+                     const int32_t* block_expert, const int32_t* num_post, int64_t num_slots, int64_t experts, int64_t block,
+                     int dtype, void* stream);
 
 #ifdef __cplusplus
 }

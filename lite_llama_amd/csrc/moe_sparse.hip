@@ -5,8 +5,8 @@
 //                     neighbours, a group's score is the sum of its two best scores, only the best `group_keep` groups stay
 //                     eligible; the `top` best eligible experts are chosen, their scores divided by their sum (+ 1e-20) and
 //                     multiplied by `route_scale`.  One more row of weights may give a per-token sigmoid scale (for a shared
-//                     expert).  One wave per token; selection by ranks (ties: the lower index first), so slot k of a token holds
-//                     its k-th best expert.
+//                     expert).  Two launches: the logits as an 8 x 8 register-tiled product per wave, then one wave per token
+//                     that selects by ranks (ties: the lower index first), so slot k of a token holds its k-th best expert.
 //   ll_moe_sort       slots (token, k) sorted by expert, every expert's run padded to the row-block size with a sentinel:
 //                     sorted_ids / block_expert / num_post as in moe_align_block_size.  Deterministic: no atomics.
 //   ll_moe_rows_gemm  the grouped products over sorted row blocks: either act = silu(a Wg_e^T) * (a Wu_e^T) (gate and up rows
@@ -32,11 +32,78 @@ __device__ __forceinline__ void stv(void* p, int64_t i, float v) {
 __device__ __forceinline__ float sigmoid_exact(float v) { return 1.0f / (1.0f + expf(-v)); }
 
 // ------------------------------------------------------------------------------------------------------------------------
-// router: one 64-thread workgroup per token.  LDS: scores [E], group score [G], group kept [G], chosen scores [top]
+// router, first launch: logits [n][experts (+ 1)] = h W^T in fp32.  A wave owns 8 tokens x 8 weight rows and walks the width
+// in pieces (16 bytes where rows are aligned): 16 piece loads feed 64 x VEC fused multiply-adds, so a weight row is fetched
+// once per 8 tokens and a token row once per 8 experts.  A token's logit does not depend on which other tokens ride along:
+// every lane sums ITS pieces in order, then the lanes are added in a fixed order.
 // ------------------------------------------------------------------------------------------------------------------------
-template <int DT>
-__global__ __launch_bounds__(64) void group_router_kernel(const void* __restrict__ h, int64_t h_ld, const void* __restrict__ w_router,
-                                                          const void* __restrict__ w_extra, int width, int experts, int top,
+template <int DT, int VEC>
+__device__ __forceinline__ void load_piece(const void* p, int64_t at, float (&o)[VEC]) {
+  if constexpr (VEC == 1) {
+    o[0] = ldv<DT>(p, at);
+  } else if constexpr (DT == LL_F32) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>((const float*)p + at);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = v[i];
+  } else {
+    const U16x8 v = *reinterpret_cast<const U16x8*>((const uint16_t*)p + at);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = to_f32<DT>(v.v[i]);
+  }
+}
+
+template <int DT, int VEC>
+__global__ __launch_bounds__(256) void router_logits_kernel(const void* __restrict__ h, int64_t h_ld, const void* __restrict__ w_router,
+                                                            const void* __restrict__ w_extra, int width, int experts, int rows,
+                                                            float* __restrict__ logits, int64_t n) {
+  constexpr int TW = 8, EW = 8;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t t0 = (int64_t)blockIdx.x * TW;
+  const int e0 = (blockIdx.y * 4 + wave) * EW;
+  if (e0 >= rows) return;   // (wave-uniform; no workgroup barrier below)
+  int64_t hat[TW];
+  const void* wp[EW];
+  int64_t wat[EW];
+#pragma unroll
+  for (int i = 0; i < TW; ++i) hat[i] = (t0 + i < n ? t0 + i : n - 1) * h_ld;
+#pragma unroll
+  for (int j = 0; j < EW; ++j) {
+    const int e = e0 + j < rows ? e0 + j : rows - 1;
+    wp[j] = e < experts ? w_router : w_extra;
+    wat[j] = e < experts ? (int64_t)e * width : 0;
+  }
+  float acc[TW][EW];
+#pragma unroll
+  for (int i = 0; i < TW; ++i)
+#pragma unroll
+    for (int j = 0; j < EW; ++j) acc[i][j] = 0.f;
+  for (int p = lane * VEC; p < width; p += 64 * VEC) {
+    float hv[TW][VEC];
+#pragma unroll
+    for (int i = 0; i < TW; ++i) load_piece<DT, VEC>(h, hat[i] + p, hv[i]);
+#pragma unroll
+    for (int j = 0; j < EW; ++j) {
+      float wv[VEC];
+      load_piece<DT, VEC>(wp[j], wat[j] + p, wv);
+#pragma unroll
+      for (int i = 0; i < TW; ++i)
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[i][j] += hv[i][k] * wv[k];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TW; ++i)
+#pragma unroll
+    for (int j = 0; j < EW; ++j) {
+      const float v = wave_sum(acc[i][j]);
+      if (lane == 0 && t0 + i < n && e0 + j < rows) logits[(t0 + i) * rows + e0 + j] = v;
+    }
+}
+
+// router, second launch: one 64-thread workgroup per token over its logits.  LDS: scores [E], group score [G], group kept
+// [G], chosen scores [top]
+template <int DUMMY>
+__global__ __launch_bounds__(64) void group_select_kernel(const float* __restrict__ logits, int rows, int experts, int top,
                                                           int group_count, int group_keep, float route_scale,
                                                           int32_t* __restrict__ ids, float* __restrict__ weights,
                                                           float* __restrict__ extra_scale) {
@@ -47,19 +114,10 @@ __global__ __launch_bounds__(64) void group_router_kernel(const void* __restrict
   float* chosen = gkeep + group_count;      // [top]
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
-  const int64_t hrow = t * h_ld;
-  for (int e = 0; e < experts + (w_extra ? 1 : 0); ++e) {
-    const bool extra = e == experts;
-    const void* wr = extra ? w_extra : w_router;
-    const int64_t wrow = extra ? 0 : (int64_t)e * width;
-    float d = 0.f;
-    for (int i = lane; i < width; i += 64) d += ldv<DT>(h, hrow + i) * ldv<DT>(wr, wrow + i);
-    d = wave_sum(d);
-    if (lane == 0) {
-      const float s = sigmoid_exact(d);
-      if (extra) extra_scale[t] = s;
-      else score[e] = s;
-    }
+  for (int e = lane; e < rows; e += 64) {
+    const float s = sigmoid_exact(logits[t * rows + e]);
+    if (e < experts) score[e] = s;
+    else extra_scale[t] = s;
   }
   __syncthreads();
   const int per = experts / group_count;
@@ -294,6 +352,106 @@ __global__ __launch_bounds__(64) void moe_rows_gemm_mfma_kernel(const uint16_t* 
   }
 }
 
+// ------------------------------------------------------------------------------------------------------------------------
+// grouped products, LDS-tiled MFMA form for prompt-sized inputs: a workgroup of four waves owns 128 sorted rows x 128 weight
+// rows (gate|up: 64 output columns, gate rows and up rows of the same columns side by side) and walks the contraction in steps
+// of 64.  Both tiles are fetched ONCE per workgroup (global -> registers -> LDS, the next step's loads in flight under the
+// products); a wave multiplies all eight row tiles with two weight tiles (its gate and its up tile), so every A fragment read
+// from LDS feeds two MFMAs and every weight fragment eight.
+// ------------------------------------------------------------------------------------------------------------------------
+template <int DT, bool GLU>
+__global__ __launch_bounds__(256) void moe_rows_gemm_tiled_kernel(const uint16_t* __restrict__ a, int64_t a_ld, int a_div,
+                                                                  const uint16_t* __restrict__ w, int64_t w_stride_e, int K, int N,
+                                                                  const float* __restrict__ slot_weight, uint16_t* __restrict__ out,
+                                                                  int64_t out_ld, const int32_t* __restrict__ sorted,
+                                                                  const int32_t* __restrict__ block_expert,
+                                                                  const int32_t* __restrict__ num_post, int num_slots) {
+  constexpr int BM = 128, WN = 128, BK = 64, STR = BK + 8, CW = GLU ? 64 : 128;
+  __shared__ __attribute__((aligned(16))) uint16_t lds_a[BM * STR];
+  __shared__ __attribute__((aligned(16))) uint16_t lds_w[WN * STR];
+  __shared__ int rows_s[BM];
+  const int block = blockIdx.x;
+  if (block * BM >= num_post[0]) return;
+  const int e = block_expert[block];
+  const int n0 = blockIdx.y * CW;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, t = lane & 15, c = lane >> 4;
+  if (tid < BM) rows_s[tid] = sorted[block * BM + tid];
+  __syncthreads();
+  const uint16_t* aptr[4];
+  const uint16_t* wptr[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int i = tid + 256 * u, row = i >> 3, pc = i & 7;
+    const int slot = rows_s[row];
+    aptr[u] = slot < num_slots ? a + (int64_t)(slot / a_div) * a_ld + 8 * pc : nullptr;
+    const int col = GLU ? n0 + (row & 63) : n0 + row;
+    const int64_t grow = (GLU && row >= 64) ? (int64_t)N + col : col;
+    wptr[u] = col < N ? w + (int64_t)e * w_stride_e + grow * K + 8 * pc : nullptr;
+  }
+  Q4 ra[4], rw[4];
+#define LL_FETCH(K0)                                                                                        \
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) {                                                           \
+    const bool in = (K0) + 8 * ((tid + 256 * u) & 7) < K;                                                   \
+    ra[u] = (in && aptr[u]) ? *reinterpret_cast<const Q4*>(aptr[u] + (K0)) : Q4{0, 0, 0, 0};                \
+    rw[u] = (in && wptr[u]) ? *reinterpret_cast<const Q4*>(wptr[u] + (K0)) : Q4{0, 0, 0, 0};                \
+  }
+#define LL_STAGE()                                                                                          \
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) {                                                           \
+    const int i = tid + 256 * u, row = i >> 3, pc = i & 7;                                                  \
+    *reinterpret_cast<Q4*>(&lds_a[row * STR + 8 * pc]) = ra[u];                                             \
+    *reinterpret_cast<Q4*>(&lds_w[row * STR + 8 * pc]) = rw[u];                                             \
+  }
+  const int tile0 = GLU ? wave : 2 * wave, tile1 = GLU ? 4 + wave : 2 * wave + 1;
+  f32x4 acc[2][8];
+#pragma unroll
+  for (int m = 0; m < 8; ++m) acc[0][m] = acc[1][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+  LL_FETCH(0)
+  LL_STAGE()
+  __syncthreads();
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    if (k0 + BK < K) { LL_FETCH(k0 + BK) }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const Q4 w0 = *reinterpret_cast<const Q4*>(&lds_w[(16 * tile0 + t) * STR + 32 * ks + 8 * c]);
+      const Q4 w1 = *reinterpret_cast<const Q4*>(&lds_w[(16 * tile1 + t) * STR + 32 * ks + 8 * c]);
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        const Q4 af = *reinterpret_cast<const Q4*>(&lds_a[(16 * m + t) * STR + 32 * ks + 8 * c]);
+        acc[0][m] = mfma16<DT>(w0, af, acc[0][m]);
+        acc[1][m] = mfma16<DT>(w1, af, acc[1][m]);
+      }
+    }
+    __syncthreads();   // everybody has read this step's tiles
+    if (k0 + BK < K) { LL_STAGE() }
+    __syncthreads();
+  }
+#undef LL_FETCH
+#undef LL_STAGE
+#pragma unroll
+  for (int m = 0; m < 8; ++m) {
+    const int slot = rows_s[16 * m + t];
+    if (slot >= num_slots) continue;
+    uint16_t* orow = out + (int64_t)slot * out_ld;
+    if (GLU) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int col = n0 + 16 * wave + 4 * c + r;
+        const float g = acc[0][m][r];
+        if (col < N) orow[col] = from_f32<DT>(g * ll_sigmoidf(g) * acc[1][m][r]);
+      }
+    } else {
+      const float sw = slot_weight ? slot_weight[slot] : 1.0f;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int col = n0 + 16 * (2 * wave + j) + 4 * c + r;
+          if (col < N) orow[col] = from_f32<DT>(acc[j][m][r] * sw);
+        }
+    }
+  }
+}
+
 }  // namespace
 
 #define LL_BY_DTYPE(dtype, CALL)             \
@@ -303,36 +461,57 @@ __global__ __launch_bounds__(64) void moe_rows_gemm_mfma_kernel(const uint16_t* 
     else { CALL(LL_F32); }                   \
   } while (0)
 
+// logits: fp32 scratch [n][experts + (w_extra ? 1 : 0)]
 extern "C" int ll_group_router(const void* h, int64_t h_ld, const void* w_router, const void* w_extra, int64_t n, int64_t width,
                                int64_t experts, int64_t top, int64_t group_count, int64_t group_keep, float route_scale,
-                               int32_t* ids, float* weights, float* extra_scale, int dtype, void* stream) {
+                               int32_t* ids, float* weights, float* extra_scale, float* logits, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
   if (n < 0 || width < 1 || h_ld < width || experts < 1 || experts > 4096 || top < 1 || top > experts || top > 64 || group_count < 1 ||
       experts % group_count || group_keep < 1 || group_keep > group_count || group_keep * (experts / group_count) < top)
     return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
-  if (!h || !w_router || !ids || !weights || (w_extra && !extra_scale)) return LL_ERR_ARG;
-  const size_t lds = sizeof(float) * (size_t)(experts + 2 * group_count + top);
+  if (!h || !w_router || !ids || !weights || !logits || (w_extra && !extra_scale)) return LL_ERR_ARG;
+  const int rows = (int)experts + (w_extra ? 1 : 0);
+  const int vec = dtype == LL_F32 ? 4 : 8;
+  const bool aligned = width % vec == 0 && h_ld % vec == 0 && ll_aligned16(h) && ll_aligned16(w_router) && (!w_extra || ll_aligned16(w_extra));
+  const dim3 grid((unsigned)((n + 7) / 8), (unsigned)((rows + 31) / 32));
   hipStream_t st = (hipStream_t)stream;
-#define CALL(DT)                                                                                                                  \
-  group_router_kernel<DT><<<dim3((unsigned)n), 64, lds, st>>>(h, h_ld, w_router, w_extra, (int)width, (int)experts, (int)top,      \
-                                                              (int)group_count, (int)group_keep, route_scale, ids, weights, extra_scale)
-  LL_BY_DTYPE(dtype, CALL);
+#define LL_RL_ARGS h, h_ld, w_router, w_extra, (int)width, (int)experts, rows, logits, n
+  if (!aligned) {
+#define CALL(DT) router_logits_kernel<DT, 1><<<grid, 256, 0, st>>>(LL_RL_ARGS)
+    LL_BY_DTYPE(dtype, CALL);
 #undef CALL
+  } else if (dtype == LL_F32) {
+    router_logits_kernel<LL_F32, 4><<<grid, 256, 0, st>>>(LL_RL_ARGS);
+  } else if (dtype == LL_F16) {
+    router_logits_kernel<LL_F16, 8><<<grid, 256, 0, st>>>(LL_RL_ARGS);
+  } else {
+    router_logits_kernel<LL_BF16, 8><<<grid, 256, 0, st>>>(LL_RL_ARGS);
+  }
+#undef LL_RL_ARGS
+  const size_t lds = sizeof(float) * (size_t)(experts + 2 * group_count + top);
+  group_select_kernel<0><<<dim3((unsigned)n), 64, lds, st>>>(logits, rows, (int)experts, (int)top, (int)group_count, (int)group_keep,
+                                                             route_scale, ids, weights, extra_scale);
   return LL_LAUNCH_CHECK();
 }
 
-extern "C" int64_t ll_moe_rows_block(void) { return 32; }
+// rows per sorted block: 128 (the LDS-tiled form) when the experts average at least 128 slots each and the 16-bit matrix-core
+// forms apply, else 32
+extern "C" int64_t ll_moe_rows_block(int64_t num_slots, int64_t experts, int64_t width, int64_t ff, int dtype) {
+  static const bool small = getenv("LL_MOE_ROWS_SMALL") != nullptr;   // A/B knob, read once
+  return (!small && dtype != LL_F32 && width % 8 == 0 && ff % 8 == 0 && num_slots >= 128 * experts) ? 128 : 32;
+}
 
 // counts: int32 scratch [experts].  sorted [num_slots + experts * (block - 1)], block_expert [ceil(that / block)], num_post [1]
-extern "C" int ll_moe_sort(const int32_t* ids, int64_t num_slots, int64_t experts, int32_t* counts, int32_t* sorted,
+extern "C" int ll_moe_sort(const int32_t* ids, int64_t num_slots, int64_t experts, int64_t block, int32_t* counts, int32_t* sorted,
                            int32_t* block_expert, int32_t* num_post, void* stream) {
-  if (num_slots < 0 || experts < 1 || experts > 65535 || num_slots + experts * 32 >= (1ll << 31)) return LL_ERR_SHAPE;
+  if (num_slots < 0 || experts < 1 || experts > 65535 || (block != 32 && block != 128) || num_slots + experts * block >= (1ll << 31))
+    return LL_ERR_SHAPE;
   if (!ids || !counts || !sorted || !block_expert || !num_post) return LL_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
   moe_count_kernel<<<dim3((unsigned)experts), 256, 0, st>>>(ids, (int)num_slots, counts);
-  moe_place_kernel<<<dim3((unsigned)experts), 256, 0, st>>>(ids, (int)num_slots, (int)experts, 32, counts, sorted, block_expert,
-                                                            num_post);
+  moe_place_kernel<<<dim3((unsigned)experts), 256, 0, st>>>(ids, (int)num_slots, (int)experts, (int)block, counts, sorted,
+                                                            block_expert, num_post);
   return LL_LAUNCH_CHECK();
 }
 
@@ -340,17 +519,30 @@ extern "C" int ll_moe_sort(const int32_t* ids, int64_t num_slots, int64_t expert
 // a[slot / a_div]; glu == 0: w [experts][N][K], out[slot][N] = (a[slot / a_div] W^T) * slot_weight[slot] (NULL: 1).
 extern "C" int ll_moe_rows_gemm(const void* a, int64_t a_ld, int64_t a_div, const void* w, int64_t w_stride_e, int64_t K, int64_t N,
                                 int glu, const float* slot_weight, void* out, int64_t out_ld, const int32_t* sorted,
-                                const int32_t* block_expert, const int32_t* num_post, int64_t num_slots, int64_t experts, int dtype,
-                                void* stream) {
+                                const int32_t* block_expert, const int32_t* num_post, int64_t num_slots, int64_t experts,
+                                int64_t block, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
-  if (num_slots < 0 || K < 1 || N < 1 || a_div < 1 || a_ld < K || out_ld < N || w_stride_e < (glu ? 2 : 1) * N * K || experts < 1)
+  if (num_slots < 0 || K < 1 || N < 1 || a_div < 1 || a_ld < K || out_ld < N || w_stride_e < (glu ? 2 : 1) * N * K || experts < 1 ||
+      (block != 32 && block != 128))
     return LL_ERR_SHAPE;
   if (num_slots == 0) return LL_OK;
   if (!a || !w || !out || !sorted || !block_expert || !num_post) return LL_ERR_ARG;
-  const int64_t max_blocks = (num_slots + experts * 31 + 31) / 32;
+  const int64_t max_blocks = (num_slots + experts * (block - 1) + block - 1) / block;
   hipStream_t st = (hipStream_t)stream;
   static const bool no_mfma = getenv("LL_MOE_ROWS_VALU") != nullptr;   // A/B knob, read once
   const bool mfma = !no_mfma && dtype != LL_F32 && K % 8 == 0 && a_ld % 8 == 0 && w_stride_e % 8 == 0 && ll_aligned16(a) && ll_aligned16(w);
+  if (block == 128) {
+    if (!mfma) return LL_ERR_SHAPE;   // (blocks of 128 rows are only sorted for the tiled matrix-core form)
+    const dim3 grid((unsigned)max_blocks, (unsigned)((N + (glu ? 63 : 127)) / (glu ? 64 : 128)));
+#define CALL_T(DT, G)                                                                                                          \
+  moe_rows_gemm_tiled_kernel<DT, G><<<grid, 256, 0, st>>>((const uint16_t*)a, a_ld, (int)a_div, (const uint16_t*)w, w_stride_e, \
+                                                          (int)K, (int)N, slot_weight, (uint16_t*)out, out_ld, sorted, block_expert, \
+                                                          num_post, (int)num_slots)
+    if (dtype == LL_F16) { if (glu) CALL_T(LL_F16, true); else CALL_T(LL_F16, false); }
+    else { if (glu) CALL_T(LL_BF16, true); else CALL_T(LL_BF16, false); }
+#undef CALL_T
+    return LL_LAUNCH_CHECK();
+  }
   if (mfma) {
     const dim3 grid((unsigned)max_blocks, (unsigned)((N + 31) / 32));
 #define CALL_M(DT, G)                                                                                                         \

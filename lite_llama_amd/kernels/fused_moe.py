@@ -267,9 +267,11 @@ def group_router(h: torch.Tensor, router_weight: torch.Tensor, top: int, group_c
     ids = torch.empty(n, top, dtype=torch.int32, device=h.device)
     weights = torch.empty(n, top, dtype=torch.float32, device=h.device)
     extra = torch.empty(n, dtype=torch.float32, device=h.device) if extra_weight is not None else None
+    logits = torch.empty(n, experts + (1 if extra_weight is not None else 0), dtype=torch.float32, device=h.device)
     L.check(L.lib().ll_group_router(h.data_ptr(), h.stride(0), router_weight.data_ptr(), L.ptr(extra_weight), n, width, experts,
                                     int(top), int(group_count), int(group_keep), float(route_scale), ids.data_ptr(),
-                                    weights.data_ptr(), L.ptr(extra), L.dtype_code(h.dtype), L.stream_ptr()), "group_router")
+                                    weights.data_ptr(), L.ptr(extra), logits.data_ptr(), L.dtype_code(h.dtype), L.stream_ptr()),
+            "group_router")
     return ids, weights, extra
 
 
@@ -292,21 +294,21 @@ def sparse_glu_experts(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.T
             or weights.shape != ids.shape:
         raise ValueError("sparse_glu_experts: int32 ids and fp32 weights [n, top]")
     lib = L.lib()
-    block = int(lib.ll_moe_rows_block())
     slots = n * top
+    block = int(lib.ll_moe_rows_block(slots, experts, width, ff, L.dtype_code(dt)))
     padded = slots + experts * (block - 1)
     meta = torch.empty(experts + padded + -(-padded // block) + 1, dtype=torch.int32, device=h.device)
     counts, sorted_ids = meta[:experts], meta[experts:experts + padded]
     block_expert, num_post = meta[experts + padded:-1], meta[-1:]
-    L.check(lib.ll_moe_sort(ids.data_ptr(), slots, experts, counts.data_ptr(), sorted_ids.data_ptr(), block_expert.data_ptr(),
+    L.check(lib.ll_moe_sort(ids.data_ptr(), slots, experts, block, counts.data_ptr(), sorted_ids.data_ptr(), block_expert.data_ptr(),
                             num_post.data_ptr(), L.stream_ptr()), "moe_sort")
     act = torch.empty(slots, ff, dtype=dt, device=h.device)
     out = torch.empty(n, top, width, dtype=dt, device=h.device)
     code, st = L.dtype_code(dt), L.stream_ptr()
     L.check(lib.ll_moe_rows_gemm(h.data_ptr(), h.stride(0), top, w_gate_up.data_ptr(), w_gate_up.stride(0), width, ff, 1, 0,
                                  act.data_ptr(), ff, sorted_ids.data_ptr(), block_expert.data_ptr(), num_post.data_ptr(), slots,
-                                 experts, code, st), "moe_rows_gemm (gate|up)")
+                                 experts, block, code, st), "moe_rows_gemm (gate|up)")
     L.check(lib.ll_moe_rows_gemm(act.data_ptr(), ff, 1, w_down.data_ptr(), w_down.stride(0), ff, width, 0, weights.data_ptr(),
                                  out.data_ptr(), width, sorted_ids.data_ptr(), block_expert.data_ptr(), num_post.data_ptr(), slots,
-                                 experts, code, st), "moe_rows_gemm (down)")
+                                 experts, block, code, st), "moe_rows_gemm (down)")
     return out

@@ -575,8 +575,13 @@ class LayeredLM(nn.Module):
                 fill(p, std=1.0 / (p.shape[1] ** 0.5))
             elif name == "embed_tokens.weight":
                 fill(p, std=1.0)
-            elif leaf in ("norm1_weight", "norm2_weight", "norm_weight", "q_norm_weight", "k_norm_weight", "out_norm_weight"):
+            elif leaf in ("norm1_weight", "norm2_weight", "norm_weight", "q_norm_weight", "k_norm_weight", "out_norm_weight",
+                          "norm1b_weight", "norm2b_weight", "kv_norm_weight"):
                 fill(p, std=0.1, mean=1.0)
+            elif leaf in ("uk_weight", "uv_weight", "router_weight", "gate_up_weight", "down_weight", "shared_scale_weight"):
+                fill(p, std=1.0 / (p.shape[-1] ** 0.5))
+            elif leaf in ("rg1_bias", "rg2_bias", "z_bias", "x_bias"):
+                fill(p, std=0.5)
             elif leaf in ("shift", "lower"):
                 fill(p, lo=0.0, hi=0.9)
             elif leaf in ("f_bias", "sink", "act", "loop_step"):

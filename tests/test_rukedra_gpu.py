@@ -67,7 +67,7 @@ def test_gated_group_norm_sums_gates_norms_adds_and_norms_again(dtype, width, gr
     pick = torch.tensor([3, 0], device=DEV)
     x3 = x[pick].contiguous()
     gated_group_norm(x3, upd.rows(pick), nw, eps, groups)
-    assert torch.equal(x3, x1[pick])
+    assert torch.allclose(x3, x1[pick], rtol=0, atol=2e-6 * float(x1.abs().max()))   # (aligned rows take the vector form)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -248,7 +248,8 @@ def test_group_router_chooses_like_the_oracle(dtype, experts, top, groups, width
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n,width,experts,top,ff", [(37, 64, 6, 3, 24), (5, 60, 9, 2, 12), (1, 96, 4, 4, 40), (300, 32, 3, 1, 8)])
+@pytest.mark.parametrize("n,width,experts,top,ff", [(37, 64, 6, 3, 24), (5, 60, 9, 2, 12), (1, 96, 4, 4, 40), (300, 32, 3, 1, 8),
+                                                    (600, 64, 3, 2, 24), (1100, 136, 4, 2, 72)])   # (the last two: blocks of 128 rows)
 def test_expert_products_per_slot(dtype, n, width, experts, top, ff):
     from lite_llama_amd.kernels.fused_moe import sparse_glu_experts
     from oracle import rukedra as O
