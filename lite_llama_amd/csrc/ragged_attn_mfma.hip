@@ -49,7 +49,8 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
     const int32_t* __restrict__ token_table, int64_t tt_stride, const int32_t* __restrict__ seq_req,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const uint16_t* __restrict__ sink,
     float scale_log2, uint16_t* __restrict__ out, float* __restrict__ partials, int max_parts, int heads, int kv_heads, int dk,
-    int dv, int64_t k_stride, int64_t v_stride, int window) {
+    int dv, int64_t k_stride, int64_t v_stride, int window, int shared_kv) {
+  static_assert(NTM / 2 == NSM, "value fragments of shared rows are the key fragments");
   constexpr int QB = 1;
   constexpr bool DECODE = true;
   constexpr int VSTR = NTM * 16 + 8;
@@ -125,8 +126,10 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
     for (int s = 0; s < NTM / 2; ++s) {
       const int ch = 8 * (4 * s + c);
       const bool in = s < nsv && ch < dv;
-      ga[s] = (in && okA) ? *reinterpret_cast<const Q4*>(vA + ch) : zero4;
-      gb[s] = (in && okB) ? *reinterpret_cast<const Q4*>(vB + ch) : zero4;
+      // shared_kv: the value rows ARE the key rows (a latent cache): the key fragments just loaded are the value fragments
+      // (channels past dv ride along into output columns that are never stored)
+      ga[s] = shared_kv ? fa[s] : (in && okA) ? *reinterpret_cast<const Q4*>(vA + ch) : zero4;
+      gb[s] = shared_kv ? fb[s] : (in && okB) ? *reinterpret_cast<const Q4*>(vB + ch) : zero4;
     }
   };
   Q4 ka[NSM], kb[NSM], va[NTM / 2], vb[NTM / 2];
@@ -276,7 +279,7 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
     const int32_t* __restrict__ token_table, int64_t tt_stride, const int32_t* __restrict__ seq_req,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const uint16_t* __restrict__ sink,
     float scale_log2, uint16_t* __restrict__ out, int heads, int kv_heads, int dk, int dv, int64_t k_stride, int64_t v_stride,
-    int window) {
+    int window, int shared_kv) {
   constexpr int KSTR = NSM * 32 + 8, VSTR = NTM * 16 + 8;
   constexpr int KPASS = (32 * NSM * 4 + 255) / 256, VPASS = (32 * NTM * 2 + 255) / 256;  // 16-byte pieces per thread
   __shared__ __attribute__((aligned(16))) uint16_t lds_k[32 * KSTR];
@@ -302,7 +305,10 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
   const int32_t* table = token_table + (int64_t)seq_req[b] * tt_stride;
   const int ns = (dk + 31) / 32, nt = (dv + 15) / 16;
   const int kcpr = dk / 8, vcpr = dv / 8;                                  // 16-byte pieces per cache row
-  const uint16_t* vtr = lds_v + (4 * c + (t >> 2)) * VSTR + (t & 3) * 4;
+  static_assert(KSTR == VSTR, "value tiles of shared rows are read from the key tile");
+  // shared_kv: the value rows ARE the key rows (a latent cache): nothing is fetched or staged for V, the transposing reads go
+  // to the key tile (channels past dv land in output columns that are never stored)
+  const uint16_t* vtr = (shared_kv ? lds_k : lds_v) + (4 * c + (t >> 2)) * VSTR + (t & 3) * 4;
 
   for (int i = tid; i < 32 * KSTR / 8; i += 256) reinterpret_cast<Q4*>(lds_k)[i] = Q4{0, 0, 0, 0};   // (pad columns stay zero)
   for (int i = tid; i < 32 * VSTR / 8; i += 256) reinterpret_cast<Q4*>(lds_v)[i] = Q4{0, 0, 0, 0};
@@ -331,7 +337,7 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
                 ? *reinterpret_cast<const Q4*>(k_cache + (int64_t)table[(P) + key] * k_stride + (int64_t)g * dk + 8 * piece) \
                 : Q4{0, 0, 0, 0};                                                                                  \
   }                                                                                                                \
-  _Pragma("unroll") for (int u = 0; u < VPASS; ++u) {                                                              \
+  if (!shared_kv) _Pragma("unroll") for (int u = 0; u < VPASS; ++u) {                                              \
     const int i = tid + 256 * u, key = i / vcpr, piece = i - key * vcpr;                                           \
     vr[u] = (key < 32 && (P) + key < k_hi)                                                                         \
                 ? *reinterpret_cast<const Q4*>(v_cache + (int64_t)table[(P) + key] * v_stride + (int64_t)g * dv + 8 * piece) \
@@ -342,7 +348,7 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
     const int i = tid + 256 * u, key = i / kcpr, piece = i - key * kcpr;                     \
     if (key < 32) *reinterpret_cast<Q4*>(&lds_k[key * KSTR + 8 * piece]) = kr[u];            \
   }                                                                                          \
-  _Pragma("unroll") for (int u = 0; u < VPASS; ++u) {                                        \
+  if (!shared_kv) _Pragma("unroll") for (int u = 0; u < VPASS; ++u) {                        \
     const int i = tid + 256 * u, key = i / vcpr, piece = i - key * vcpr;                     \
     if (key < 32) *reinterpret_cast<Q4*>(&lds_v[key * VSTR + 8 * piece]) = vr[u];            \
   }
@@ -485,6 +491,7 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
   const int max_parts = decode ? (int)((longest_context + kPart - 1) / kPart) : 1;
   if (decode && max_parts > 1 && !partials) return LL_ERR_ARG;
   const int group = (int)(heads / kv_heads);
+  const int shared_kv = (v_cache == k_cache && v_stride == k_stride && kv_heads == 1) ? 1 : 0;   // a latent cache: values = leading key columns
   const dim3 grid((unsigned)max_parts, (unsigned)(kv_heads * ((group + 15) / 16)), (unsigned)batch);
   hipStream_t st = (hipStream_t)stream;
   const float scale_log2 = scale * kLog2e;
@@ -492,7 +499,7 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
   ragged_attention_mfma_decode_kernel<DT, NS, NT><<<grid, 64, 0, st>>>(                                                      \
       (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, token_table, tt_stride, seq_req, seq_start,    \
       seq_first_pos, (const uint16_t*)sink, scale_log2, (uint16_t*)out, partials, max_parts, (int)heads, (int)kv_heads, (int)dk, \
-      (int)dv, k_stride, v_stride, (int)window)
+      (int)dv, k_stride, v_stride, (int)window, shared_kv)
 #define CALL(DT)                                         \
   if (dk <= 64 && dv <= 64) { CALL_D(DT, 2, 4); }        \
   else if (dk <= 128 && dv <= 128) { CALL_D(DT, 4, 8); } \
@@ -503,7 +510,7 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
   ragged_attention_mfma_prefill4_kernel<DT, NS, NT><<<grid4, 256, 0, st>>>(                                                 \
       (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, token_table, tt_stride, seq_req, seq_start,   \
       seq_first_pos, (const uint16_t*)sink, scale_log2, (uint16_t*)out, (int)heads, (int)kv_heads, (int)dk, (int)dv, k_stride,   \
-      v_stride, (int)window)
+      v_stride, (int)window, shared_kv)
 #define CALL_P(DT)                                       \
   if (dk <= 64 && dv <= 64) { CALL_4(DT, 2, 4); }        \
   else if (dk <= 128 && dv <= 128) { CALL_4(DT, 4, 8); } \

@@ -55,8 +55,8 @@ class RotarySpec:
     base: float
     factor: float = 0.0         # 0: no scaling
     original: float = 0.0       # positions the unscaled frequencies were made for
-    fast: float = 32.0          # turns over `original` positions above which a pair keeps its frequency
-    slow: float = 1.0           # ... and below which it is divided by `factor`
+    fast: float = 0.0           # turns over `original` positions above which a pair keeps its frequency
+    slow: float = 0.0           # ... and below which it is divided by `factor`
 
     def table(self) -> tuple[list[float], float]:
         """``(frequency per pair, amplitude of cos / sin)``."""
@@ -78,9 +78,11 @@ class RotarySpec:
 
     @staticmethod
     def from_config(rot: Mapping) -> "RotarySpec":
-        sc = rot.get("scaling") or {}
-        return RotarySpec(int(rot["dims"]), float(rot["base"]), float(sc.get("factor", 0.0)), float(sc.get("original", 0.0)),
-                          float(sc.get("fast", 32.0)), float(sc.get("slow", 1.0)))
+        sc = rot.get("scaling")
+        if not sc:
+            return RotarySpec(int(rot["dims"]), float(rot["base"]))
+        return RotarySpec(int(rot["dims"]), float(rot["base"]), float(sc["factor"]), float(sc["original"]), float(sc["fast"]),
+                          float(sc["slow"]))
 
 
 @dataclass(frozen=True)
