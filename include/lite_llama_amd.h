@@ -631,10 +631,13 @@ int ll_glu_act(void* out, const void* gate, int64_t gate_ld, const void* up, int
 int ll_softcap(void* x, int64_t n, float cap, int dtype, void* stream);
 /* minGRU: rows [z | x | g] (three pointers, one stride ld): z = sigmoid(z_raw + z_bias), u = x_raw + x_bias, candidate u + 1/2
  * (u >= 0) or sigmoid(u); S <- (1 - z) S + z candidate per channel, out = S * silu(g_raw).  state [slots][width] fp32 (read when
- * seq_first_pos > 0, written at the end of the run). */
+ * seq_first_pos > 0, written at the end of the run).  With scratch (fp32, ll_mingru_scan_scratch_floats(...) floats, > 0 for
+ * runs of 128 tokens and more; longest_run = most tokens a sequence brings) runs are walked in chunks of 32 tokens side by
+ * side: chunk maps, entering states, then the chunks again. */
+int64_t ll_mingru_scan_scratch_floats(int64_t batch, int64_t width, int64_t longest_run);
 int ll_mingru_scan(const void* z, const void* x, const void* g, int64_t ld, const void* z_bias, const void* x_bias,
                    void* out, int64_t batch, int64_t width, const int32_t* seq_start, const int32_t* seq_first_pos,
-                   const int32_t* seq_slot, float* state, int dtype, void* stream);
+                   const int32_t* seq_slot, float* state, int64_t longest_run, float* scratch, int dtype, void* stream);
 
 /* ---- attention over a shared latent (csrc/latent_attn.hip) ------------------------------------------------------------------
  * ll_latent_kv_prep: rows (stride ld) hold the latent [rank] and the rotated key part [rot] at column kv_off: the cache row

@@ -542,6 +542,82 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(const void* __restrict
   *slot = S;
 }
 
+// Chunked form of the minGRU scan for long runs.  The walk above keeps one wave per 64 channels of a sequence busy for the
+// whole run; here a run is cut into chunks of kGruChunk tokens that are walked side by side:
+//   pass 1   thread per (sequence, chunk, channel): the chunk's map S -> A S + B (A = product of (1 - z), B = the chunk walked
+//            from a zero state), into scratch
+//   pass 2   thread per (sequence, channel): the state that enters every chunk (S <- A S + B, chunk by chunk), the final state
+//            into the slot
+//   pass 3   thread per (sequence, chunk, channel): the chunk walked again from its entering state, outputs written
+// Inside a chunk the expression is the token-by-token one; across chunks the state passes through A S + B (one more rounding
+// per chunk than the plain walk).
+constexpr int kGruChunk = 32;
+
+template <int DT>
+__device__ __forceinline__ void mingru_gates(float zr, float xr, float zb, float xb, float& zt, float& cand) {
+  zt = 1.0f / (1.0f + expf(-(zr + zb)));
+  const float u = xr + xb;
+  cand = u >= 0.f ? u + 0.5f : 1.0f / (1.0f + expf(-u));
+}
+
+template <int DT, int PASS>
+__global__ __launch_bounds__(256) void mingru_chunk_kernel(const void* __restrict__ z, const void* __restrict__ x,
+                                                           const void* __restrict__ g, int64_t ld, const void* __restrict__ z_bias,
+                                                           const void* __restrict__ x_bias, void* __restrict__ out, int width,
+                                                           const int32_t* __restrict__ seq_start, int max_chunks,
+                                                           float* __restrict__ scratch) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= width) return;
+  const int b = blockIdx.y / max_chunks, k = blockIdx.y - b * max_chunks;
+  const int start = seq_start[b] + k * kGruChunk, stop_run = seq_start[b + 1];
+  if (start >= stop_run) return;
+  const int stop = start + kGruChunk < stop_run ? start + kGruChunk : stop_run;
+  const float zb = z_bias ? ldv<DT>(z_bias, c) : 0.f, xb = x_bias ? ldv<DT>(x_bias, c) : 0.f;
+  float* rec = scratch + ((int64_t)blockIdx.y * width + c) * 2;
+  if (PASS == 1) {
+    float A = 1.0f, B = 0.f;
+    for (int t = start; t < stop; ++t) {
+      const int64_t at = (int64_t)t * ld + c;
+      float zt, cand;
+      mingru_gates<DT>(ldv<DT>(z, at), ldv<DT>(x, at), zb, xb, zt, cand);
+      A = (1.0f - zt) * A;
+      B = (1.0f - zt) * B + zt * cand;
+    }
+    rec[0] = A;
+    rec[1] = B;
+  } else {
+    float S = rec[0];   // (pass 2 left the entering state here)
+    for (int t = start; t < stop; ++t) {
+      const int64_t at = (int64_t)t * ld + c;
+      float zt, cand;
+      mingru_gates<DT>(ldv<DT>(z, at), ldv<DT>(x, at), zb, xb, zt, cand);
+      S = (1.0f - zt) * S + zt * cand;
+      const float gr = ldv<DT>(g, at);
+      stv<DT>(out, (int64_t)t * width + c, S * (gr / (1.0f + expf(-gr))));
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void mingru_carry_kernel(int width, const int32_t* __restrict__ seq_start,
+                                                           const int32_t* __restrict__ seq_first_pos,
+                                                           const int32_t* __restrict__ seq_slot, float* __restrict__ state,
+                                                           int max_chunks, float* __restrict__ scratch) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= width) return;
+  const int b = blockIdx.y;
+  const int count = seq_start[b + 1] - seq_start[b];
+  const int chunks = (count + kGruChunk - 1) / kGruChunk;
+  float* slot = state + (int64_t)seq_slot[b] * width + c;
+  float S = seq_first_pos[b] > 0 ? *slot : 0.f;
+  for (int k = 0; k < chunks; ++k) {
+    float* rec = scratch + (((int64_t)b * max_chunks + k) * width + c) * 2;
+    const float A = rec[0], B = rec[1];
+    rec[0] = S;
+    S = A * S + B;
+  }
+  if (count > 0) *slot = S;
+}
+
 }  // namespace
 
 #define LL_BY_DTYPE(dtype, CALL)             \
@@ -678,15 +754,33 @@ extern "C" int ll_gated_linear_scan(const void* q, const void* f, const void* v,
   return LL_LAUNCH_CHECK();
 }
 
+extern "C" int64_t ll_mingru_scan_scratch_floats(int64_t batch, int64_t width, int64_t longest_run) {
+  static const bool plain = getenv("LL_MINGRU_PLAIN") != nullptr;   // A/B knob, read once
+  if (plain || longest_run < 4 * kGruChunk || batch < 1) return 0;   // short runs: the plain walk
+  return batch * ((longest_run + kGruChunk - 1) / kGruChunk) * width * 2;
+}
+
+// scratch: fp32, ll_mingru_scan_scratch_floats(batch, width, longest_run) floats (NULL or longest_run = 0: the plain walk)
 extern "C" int ll_mingru_scan(const void* z, const void* x, const void* g, int64_t ld, const void* z_bias, const void* x_bias,
                               void* out, int64_t batch, int64_t width, const int32_t* seq_start, const int32_t* seq_first_pos,
-                              const int32_t* seq_slot, float* state, int dtype, void* stream) {
+                              const int32_t* seq_slot, float* state, int64_t longest_run, float* scratch, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
-  if (batch < 0 || batch > 65535 || width < 1 || ld < width) return LL_ERR_SHAPE;
+  if (batch < 0 || batch > 65535 || width < 1 || ld < width || longest_run < 0) return LL_ERR_SHAPE;
   if (batch == 0) return LL_OK;
   if (!z || !x || !g || !out || !seq_start || !seq_first_pos || !seq_slot || !state) return LL_ERR_ARG;
-  const dim3 grid((unsigned)((width + 255) / 256), (unsigned)batch);
   hipStream_t st = (hipStream_t)stream;
+  const int64_t max_chunks = (longest_run + kGruChunk - 1) / kGruChunk;
+  if (scratch && ll_mingru_scan_scratch_floats(batch, width, longest_run) > 0 && batch * max_chunks <= 65535) {
+    const dim3 grid_c((unsigned)((width + 255) / 256), (unsigned)(batch * max_chunks)), grid_b((unsigned)((width + 255) / 256), (unsigned)batch);
+#define CALL(DT)                                                                                                                \
+  mingru_chunk_kernel<DT, 1><<<grid_c, 256, 0, st>>>(z, x, g, ld, z_bias, x_bias, out, (int)width, seq_start, (int)max_chunks, scratch); \
+  mingru_carry_kernel<<<grid_b, 256, 0, st>>>((int)width, seq_start, seq_first_pos, seq_slot, state, (int)max_chunks, scratch);         \
+  mingru_chunk_kernel<DT, 2><<<grid_c, 256, 0, st>>>(z, x, g, ld, z_bias, x_bias, out, (int)width, seq_start, (int)max_chunks, scratch)
+    LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return LL_LAUNCH_CHECK();
+  }
+  const dim3 grid((unsigned)((width + 255) / 256), (unsigned)batch);
 #define CALL(DT) \
   mingru_scan_kernel<DT><<<grid, 256, 0, st>>>(z, x, g, ld, z_bias, x_bias, out, (int)width, seq_start, seq_first_pos, seq_slot, state)
   LL_BY_DTYPE(dtype, CALL);

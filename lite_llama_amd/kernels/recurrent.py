@@ -68,7 +68,11 @@ def mingru_scan(zxg: torch.Tensor, width: int, z_bias, x_bias, step, state: torc
         raise ValueError("mingru_scan: the step describes another number of tokens")
     out = torch.empty(n, width, dtype=dt, device=zxg.device)
     es, base = zxg.element_size(), zxg.data_ptr()
+    # long runs: chunks of a run are walked side by side (chunk maps, entering states, the chunks again) over an fp32 scratch
+    floats = int(L.lib().ll_mingru_scan_scratch_floats(step.num_seqs, width, step.longest_run))
+    scratch = torch.empty(floats, dtype=torch.float32, device=zxg.device) if floats else None
     L.check(L.lib().ll_mingru_scan(base, base + width * es, base + 2 * width * es, zxg.stride(0), L.ptr(z_bias), L.ptr(x_bias),
                                    out.data_ptr(), step.num_seqs, width, step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(),
-                                   step.seq_slot.data_ptr(), state.data_ptr(), L.dtype_code(dt), L.stream_ptr()), "mingru_scan")
+                                   step.seq_slot.data_ptr(), state.data_ptr(), step.longest_run, L.ptr(scratch), L.dtype_code(dt),
+                                   L.stream_ptr()), "mingru_scan")
     return out

@@ -124,12 +124,17 @@ def test_latent_rows_are_normed_rotated_at_their_positions_and_written_to_their_
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width", [40, 30, 300])
-def test_mingru_carries_state_across_steps_and_ignores_stale_slots(dtype, width):
+@pytest.mark.parametrize("long", [False, True])
+def test_mingru_carries_state_across_steps_and_ignores_stale_slots(dtype, width, long):
+    """Short runs take the plain walk; runs of 128 tokens and more are walked in chunks of 32 side by side (a last chunk of 8
+    and of 22 tokens, a neighbour that brings 1 or 3 tokens into the same launch and carries its state through it)."""
     from lite_llama_amd.kernels.recurrent import mingru_scan
     from oracle import rukedra as O
 
     torch.manual_seed(width)
-    lens = {1: 23, 0: 11}
+    lens = {1: 353, 0: 154} if long else {1: 23, 0: 11}
+    plans = {False: [[(1, 0, 9), (0, 0, 1)], [(0, 1, 1), (1, 9, 1)], [(1, 10, 13), (0, 2, 9)]],
+             True: [[(1, 0, 200), (0, 0, 1)], [(1, 200, 3), (0, 1, 150)], [(0, 151, 3), (1, 203, 150)]]}
     rows = {s: _rt(torch.randn(n, 3 * width + 7, device=DEV) * 2, dtype) for s, n in lens.items()}
     zb, xb = _rt(torch.randn(width, device=DEV), dtype), _rt(torch.randn(width, device=DEV), dtype)
     eye = torch.eye(width, dtype=F64)
@@ -141,7 +146,7 @@ def test_mingru_carries_state_across_steps_and_ignores_stale_slots(dtype, width)
              "g": torch.cat([torch.zeros(width, 2 * width, dtype=F64), eye, torch.zeros(width, 7, dtype=F64)], 1), "o": eye}
         want[s] = O.mingru(r64, w, "")
     state = torch.full((3, width), 7.0, device=DEV)                     # stale: a sequence that starts must not read it
-    plan = [[(1, 0, 9), (0, 0, 1)], [(0, 1, 1), (1, 9, 1)], [(1, 10, 13), (0, 2, 9)]]
+    plan = plans[long]
     got = {s: [] for s in lens}
     for seqs in plan:
         step = _step([(s, f, c, 0) for s, f, c in seqs])
