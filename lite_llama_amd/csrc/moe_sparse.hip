@@ -32,7 +32,8 @@ __device__ __forceinline__ void stv(void* p, int64_t i, float v) {
 __device__ __forceinline__ float sigmoid_exact(float v) { return 1.0f / (1.0f + expf(-v)); }
 
 // ------------------------------------------------------------------------------------------------------------------------
-// router, first launch: logits [n][experts (+ 1)] = h W^T in fp32.  A wave owns 8 tokens x 8 weight rows and walks the width
+// router, first launch: logits [n][experts (+ 1)] = h W^T in fp32.  A wave owns 8 tokens x 8 weight rows (x 2 rows for steps of
+// a few tokens, where more and shorter waves matter more than reuse) and walks the width
 // in pieces (16 bytes where rows are aligned): 16 piece loads feed 64 x VEC fused multiply-adds, so a weight row is fetched
 // once per 8 tokens and a token row once per 8 experts.  A token's logit does not depend on which other tokens ride along:
 // every lane sums ITS pieces in order, then the lanes are added in a fixed order.
@@ -52,11 +53,11 @@ __device__ __forceinline__ void load_piece(const void* p, int64_t at, float (&o)
   }
 }
 
-template <int DT, int VEC>
+template <int DT, int VEC, int EW>
 __global__ __launch_bounds__(256) void router_logits_kernel(const void* __restrict__ h, int64_t h_ld, const void* __restrict__ w_router,
                                                             const void* __restrict__ w_extra, int width, int experts, int rows,
                                                             float* __restrict__ logits, int64_t n) {
-  constexpr int TW = 8, EW = 8;
+  constexpr int TW = 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t t0 = (int64_t)blockIdx.x * TW;
   const int e0 = (blockIdx.y * 4 + wave) * EW;
@@ -314,18 +315,29 @@ __global__ __launch_bounds__(64) void moe_rows_gemm_mfma_kernel(const uint16_t* 
   f32x4 acc[NW][2];
 #pragma unroll
   for (int j = 0; j < NW; ++j) acc[j][0] = acc[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < K; k0 += 32) {
+  // the fragments of the next two contraction steps are requested before the products of the current one: with a handful of
+  // rows per expert (decoding) the launch streams every weight row once, and only loads in flight hide that latency
+  constexpr int AHEAD = 2;
+  Q4 af[AHEAD + 1][2], wf[AHEAD + 1][NW];
+  auto fetch = [&](int k0, Q4 (&fa)[2], Q4 (&fw)[NW]) {
     const int ch = k0 + 8 * c;
     const bool in = ch < K;
-    Q4 af[2], wf[NW];
 #pragma unroll
-    for (int m = 0; m < 2; ++m) af[m] = (in && arow[m]) ? *reinterpret_cast<const Q4*>(arow[m] + ch) : Q4{0, 0, 0, 0};
+    for (int m = 0; m < 2; ++m) fa[m] = (in && arow[m]) ? *reinterpret_cast<const Q4*>(arow[m] + ch) : Q4{0, 0, 0, 0};
 #pragma unroll
-    for (int j = 0; j < NW; ++j) wf[j] = (in && wrow[j]) ? *reinterpret_cast<const Q4*>(wrow[j] + ch) : Q4{0, 0, 0, 0};
+    for (int j = 0; j < NW; ++j) fw[j] = (in && wrow[j]) ? *reinterpret_cast<const Q4*>(wrow[j] + ch) : Q4{0, 0, 0, 0};
+  };
 #pragma unroll
-    for (int j = 0; j < NW; ++j) {
-      acc[j][0] = mfma16<DT>(wf[j], af[0], acc[j][0]);
-      acc[j][1] = mfma16<DT>(wf[j], af[1], acc[j][1]);
+  for (int a2 = 0; a2 < AHEAD; ++a2) fetch(32 * a2, af[a2], wf[a2]);
+  for (int k0 = 0; k0 < K; k0 += 32 * (AHEAD + 1)) {
+#pragma unroll
+    for (int u = 0; u <= AHEAD; ++u) {   // (slot u holds step k0 + 32 u; the slot just freed receives step + AHEAD)
+      fetch(k0 + 32 * (u + AHEAD), af[(u + AHEAD) % (AHEAD + 1)], wf[(u + AHEAD) % (AHEAD + 1)]);
+#pragma unroll
+      for (int j = 0; j < NW; ++j) {
+        acc[j][0] = mfma16<DT>(wf[u][j], af[u][0], acc[j][0]);
+        acc[j][1] = mfma16<DT>(wf[u][j], af[u][1], acc[j][1]);
+      }
     }
   }
 #pragma unroll
@@ -474,20 +486,25 @@ extern "C" int ll_group_router(const void* h, int64_t h_ld, const void* w_router
   const int rows = (int)experts + (w_extra ? 1 : 0);
   const int vec = dtype == LL_F32 ? 4 : 8;
   const bool aligned = width % vec == 0 && h_ld % vec == 0 && ll_aligned16(h) && ll_aligned16(w_router) && (!w_extra || ll_aligned16(w_extra));
-  const dim3 grid((unsigned)((n + 7) / 8), (unsigned)((rows + 31) / 32));
+  const int ew = n >= 512 ? 8 : 2;   // weight rows per wave
+  const dim3 grid((unsigned)((n + 7) / 8), (unsigned)((rows + 4 * ew - 1) / (4 * ew)));
   hipStream_t st = (hipStream_t)stream;
 #define LL_RL_ARGS h, h_ld, w_router, w_extra, (int)width, (int)experts, rows, logits, n
+#define LL_RL(DT, V)                                                                         \
+  if (ew == 8) router_logits_kernel<DT, V, 8><<<grid, 256, 0, st>>>(LL_RL_ARGS);             \
+  else router_logits_kernel<DT, V, 2><<<grid, 256, 0, st>>>(LL_RL_ARGS)
   if (!aligned) {
-#define CALL(DT) router_logits_kernel<DT, 1><<<grid, 256, 0, st>>>(LL_RL_ARGS)
+#define CALL(DT) LL_RL(DT, 1)
     LL_BY_DTYPE(dtype, CALL);
 #undef CALL
   } else if (dtype == LL_F32) {
-    router_logits_kernel<LL_F32, 4><<<grid, 256, 0, st>>>(LL_RL_ARGS);
+    LL_RL(LL_F32, 4);
   } else if (dtype == LL_F16) {
-    router_logits_kernel<LL_F16, 8><<<grid, 256, 0, st>>>(LL_RL_ARGS);
+    LL_RL(LL_F16, 8);
   } else {
-    router_logits_kernel<LL_BF16, 8><<<grid, 256, 0, st>>>(LL_RL_ARGS);
+    LL_RL(LL_BF16, 8);
   }
+#undef LL_RL
 #undef LL_RL_ARGS
   const size_t lds = sizeof(float) * (size_t)(experts + 2 * group_count + top);
   group_select_kernel<0><<<dim3((unsigned)n), 64, lds, st>>>(logits, rows, (int)experts, (int)top, (int)group_count, (int)group_keep,

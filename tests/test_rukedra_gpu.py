@@ -200,6 +200,17 @@ def _window_case(dtype, heads, rank, rot, total, plan, window, hot=None, scale=0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [0, 50])
+def test_latent_rows_wider_than_the_matrix_core_forms_serve(dtype, window):
+    """A latent of 272 + 16 entries per row (more than the 16-bit matrix-core forms take): the plain form with eight value
+    columns per lane, prompt portion and decoded tokens."""
+    total = 90
+    plan = [[(1, 0, 70), (0, 0, 2)]] + [[(1, 70 + i, 1), (0, 2 + i, 1)] for i in range(20)]
+    got, want = _window_case(dtype, 2, 272, 16, total, plan, window, hot=33, scale=0.15)
+    _close(got, want, 5e-5 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rank,rot", [(40, 8), (22, 4)])             # (26 entries per row: the 16-bit matrix-core form does not apply)
 @pytest.mark.parametrize("hot", [0, 3, 63, 64, 255, 256, 600])
 def test_one_far_key_reaches_prompt_portions_and_decoded_tokens(dtype, rank, rot, hot):
@@ -231,7 +242,7 @@ def test_window_edge_in_prompts_and_in_decoding(dtype, rank, rot, window, hot):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("experts,top,groups,width", [(6, 3, (3, 2), 96), (9, 2, (3, 1), 60), (4, 2, None, 33), (64, 6, (8, 3), 128),
-                                                      (1, 1, None, 16), (8, 8, (2, 2), 40)])
+                                                      (1, 1, None, 16), (8, 8, (2, 2), 40), (5, 2, (5, 3), 24)])   # (the last: groups of one)
 def test_group_router_chooses_like_the_oracle(dtype, experts, top, groups, width):
     from lite_llama_amd.kernels.fused_moe import group_router
     from oracle import rukedra as O
