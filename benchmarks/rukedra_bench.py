@@ -106,6 +106,18 @@ def kernel_table(dev, dtype, width, heads, dim, rot, vdim, rank, ff, gru, expert
                     like = _entry("flash_decoding (head width 128, one K/V head per query head)", t_old,
                                   ctx_rows * 2 * heads * 128 * es, batch * heads * 4.0 * 128 * length)
             out.append(dict(_entry(name, t_new, nbytes, flops, like), phase=phase))
+            like_causal = like if not win else like_causal
+        if phase == "prefill":   # whole prompts: keys / values expanded per head from the step's own latents (the model's prompt form)
+            import dataclasses
+
+            qf = torch.randn(n, heads, dim + rot, device=dev).to(dtype)
+            kf = torch.randn(n, heads, dim + rot, device=dev).to(dtype)
+            vf = torch.randn(n, heads, vdim, device=dev).to(dtype)
+            own = dataclasses.replace(step, seq_slot=torch.arange(batch, dtype=torch.int32, device=dev))
+            t_new = _time(lambda: ragged_attention(qf, kf, vf, 0.1, own, table), iters=5)
+            pairs = batch * length * (length + 1) / 2
+            out.append(dict(_entry("ragged_attention (expanded keys / values, causal: the prompt form of whole prompts)", t_new,
+                                   n * heads * (2 * (dim + rot) + 2 * vdim) * es, heads * 2.0 * (dim + rot + vdim) * pairs, like_causal), phase=phase))
         # recurrence vs the framework's other recurrent layer (HGRN2 at the same number of channels)
         zxg = torch.randn(n, 3 * gru + width, device=dev).to(dtype)
         st = torch.zeros(batch, gru, device=dev)

@@ -70,10 +70,11 @@ __global__ __launch_bounds__(256) void latent_kv_prep_kernel(
 }
 
 // thread per (token, head, entry of the rotated part): q [n, heads, head_ld-strided] -> out[(t * heads + h) * out_ld + out_off + j]
+// (out may be q: a pair is read and written by the same thread)
 template <int DT>
-__global__ __launch_bounds__(256) void rotate_pairs_kernel(const void* __restrict__ q, int64_t q_tok_stride, int64_t q_head_stride,
+__global__ __launch_bounds__(256) void rotate_pairs_kernel(const void* q, int64_t q_tok_stride, int64_t q_head_stride,
                                                            int64_t q_off, int rot, const float* __restrict__ freq, int pairs,
-                                                           float amp, const int32_t* __restrict__ tok_pos, void* __restrict__ out,
+                                                           float amp, const int32_t* __restrict__ tok_pos, void* out,
                                                            int64_t out_head_stride, int64_t out_off, int64_t n, int heads) {
   const int half = (rot + 1) / 2;   // one thread per pair (or per single trailing entry)
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;

@@ -36,6 +36,7 @@ class RaggedStep:
     seq_parity: torch.Tensor
     longest_run: int = 0       # most tokens a sequence brings (host copy; 0: not known)
     longest_context: int = 0   # longest sequence after this step (host copy; 0: not known)
+    all_start: bool = False    # every sequence of the step starts at position 0 (host copy; False: not known)
 
     @property
     def seq_req(self) -> torch.Tensor:
@@ -75,6 +76,7 @@ class RaggedRunner:
         self._free_slots = list(range(max_requests))
         self._len: dict[int, int] = {}
         self._parity: dict[int, int] = {}
+        self._all_start = False    # the step planned last: every sequence at position 0
         # captured decode steps (opt-in): one hipGraph per (slots riding, context partitions) cell, see _decode_cell
         self.capture_decode = bool(capture_decode)
         self._cells: dict[tuple, "_DecodeCell"] = {}
@@ -143,6 +145,7 @@ class RaggedRunner:
         for s, n in zip(slots, new_len):
             self._len[s] = n
             self._parity[s] ^= 1
+        self._all_start = not any(first)
         return parts, longest, max(new_len)
 
     @staticmethod
@@ -166,7 +169,7 @@ class RaggedRunner:
         select = rows.reshape(-1)[v_pick].contiguous() if longest > 1 else rows.reshape(-1)
         step = RaggedStep(num_tokens=v_tokens.numel(), num_seqs=num_seqs, tok_seq=v_tok_seq, tok_pos=v_tok_pos, select=select,
                           seq_start=v_starts, seq_first_pos=v_first, seq_slot=v_slots, seq_parity=v_parity, longest_run=longest,
-                          longest_context=longest_context)
+                          longest_context=longest_context, all_start=self._all_start and longest > 1)
         return step, v_tokens
 
     @torch.no_grad()

@@ -386,7 +386,8 @@ def latent_kv_prep(rows, kv_off: int, rank: int, rot: int, kv_norm_weight, eps: 
 @torch.no_grad()
 def rotate_pairs(q, q_off: int, rot: int, freq, pairs: int, amp: float, step, out, out_off: int):
     """``q [n, heads, w]`` (unit inner stride): the ``rot`` entries at ``q_off`` of every head, rotated pair by pair at the
-    token's position, land at ``out[n, heads, w'][..., out_off : out_off + rot]`` (``out`` contiguous)."""
+    token's position, land at ``out[n, heads, w'][..., out_off : out_off + rot]`` (``out`` contiguous; it may be ``q`` itself
+    with ``out_off == q_off``: every pair is read and written by one thread)."""
     L.require_cuda(q, out, freq)
     n, heads = q.shape[0], q.shape[1]
     if q.dim() != 3 or out.dim() != 3 or q.stride(2) != 1 or not out.is_contiguous() or out.shape[:2] != q.shape[:2] \

@@ -29,6 +29,7 @@ from __future__ import annotations
 
 import math
 from collections.abc import Mapping
+import dataclasses
 from dataclasses import dataclass, field
 
 import torch
@@ -340,6 +341,9 @@ class LatentAttention(nn.Module):
     def cache_run(self) -> dict:
         return {"kind": "latent", "rank": self.spec.kv_rank, "rot": self.spec.rot_dim}
 
+    # whole prompts of at least this many tokens take the expanded form (keys / values per head from the step's own latents)
+    expand_min_run = 64
+
     def forward(self, h, step, cache, run: int, token_table):
         s = self.spec
         n = h.shape[0]
@@ -347,23 +351,54 @@ class LatentAttention(nn.Module):
         k_cache, v_cache = cache.kv_buffer[run]
         if self._freq is None or self._freq.device != h.device:
             self._freq = torch.tensor(self._freq_values, dtype=torch.float64).to(torch.float32).to(h.device)
+        cache_rows = k_cache.view(k_cache.shape[0], -1)
         c_q = latent_kv_prep(rows, self.kv_off, s.kv_rank, s.rot_dim, self.kv_norm_weight, self.eps, self._freq, self.pairs, self.amp,
-                             step, k_cache.view(k_cache.shape[0], -1), q_off=0, q_rank=s.q_rank,
-                             q_norm_weight=self.q_norm_weight if s.q_rank else None)
+                             step, cache_rows, q_off=0, q_rank=s.q_rank, q_norm_weight=self.q_norm_weight if s.q_rank else None)
         q = (self.uq_proj(c_q) if s.q_rank else rows[:, :self.q_width]).view(n, s.heads, s.dim + s.rot_dim)
-        qa = torch.empty(n, s.heads, s.kv_rank + s.rot_dim, dtype=h.dtype, device=h.device)
+        if step.all_start and step.longest_run >= self.expand_min_run:
+            o = self._expanded(q, cache_rows, step)
+        else:
+            o = self._absorbed(q, k_cache, v_cache, step, token_table)
+        if s.out_gate:
+            o = glu_act(rows[:, self.gate_off:], s.heads * s.vdim, "sigmoid", up=o)
+        return self.o_proj(o), (rows[:, self.extra_off:] if self.extra else None)
+
+    def _absorbed(self, q, k_cache, v_cache, step, token_table):
+        """Any step: queries against the cached latent rows."""
+        s, n = self.spec, q.shape[0]
+        qa = torch.empty(n, s.heads, s.kv_rank + s.rot_dim, dtype=q.dtype, device=q.device)
         # absorbed query: [heads, n, dim] x [heads, dim, rank] straight into the front columns of the query rows
         torch.bmm(q[:, :, :s.dim].transpose(0, 1), self.uk_weight.view(s.heads, s.dim, s.kv_rank),
                   out=qa[:, :, :s.kv_rank].transpose(0, 1))
         rotate_pairs(q, s.dim, s.rot_dim, self._freq, self.pairs, self.amp, step, qa, s.kv_rank)
         o_lat = ragged_attention(qa, k_cache, v_cache, s.scale, step, token_table, window=s.window)     # [n, heads * rank]
-        o = torch.empty(n, s.heads, s.vdim, dtype=h.dtype, device=h.device)
+        o = torch.empty(n, s.heads, s.vdim, dtype=q.dtype, device=q.device)
         torch.bmm(o_lat.view(n, s.heads, s.kv_rank).transpose(0, 1), self.uv_weight.view(s.heads, s.vdim, s.kv_rank).transpose(1, 2),
                   out=o.transpose(0, 1))
-        o = o.view(n, s.heads * s.vdim)
-        if s.out_gate:
-            o = glu_act(rows[:, self.gate_off:], s.heads * s.vdim, "sigmoid", up=o)
-        return self.o_proj(o), (rows[:, self.extra_off:] if self.extra else None)
+        return o.view(n, s.heads * s.vdim)
+
+    def _expanded(self, q, cache_rows, step):
+        """A step in which every sequence starts at position 0 (whole prompts): all keys a token may see are tokens of this
+        step, so keys ``[W_uk c | rotated part]`` and values ``W_uv c`` are expanded per head from the rows the step has just
+        written, and attention runs with the heads' own narrow widths (dim + rot_dim, vdim) instead of rank + rot_dim, rank:
+        a fraction of the absorbed form's work per (query, key) pair.  Same values up to rounding."""
+        s, n = self.spec, q.shape[0]
+        written = cache_rows.index_select(0, step.select.long())                        # [n, rank + rot]: normed latent | rotated part
+        latent = written[:, :s.kv_rank]
+        if q.is_contiguous():
+            qf = q
+        else:
+            qf = q.contiguous()
+        rotate_pairs(qf, s.dim, s.rot_dim, self._freq, self.pairs, self.amp, step, qf, s.dim)             # (in place)
+        keys = torch.empty(n, s.heads, s.dim + s.rot_dim, dtype=q.dtype, device=q.device)
+        keys[:, :, :s.dim] = torch.nn.functional.linear(latent, self.uk_weight).view(n, s.heads, s.dim)
+        keys[:, :, s.dim:] = written[:, None, s.kv_rank:]
+        values = torch.nn.functional.linear(latent, self.uv_weight).view(n, s.heads, s.vdim)
+        # the step's own tokens as a cache: sequence i of the step owns rows seq_start[i] .. ; positions are row offsets
+        own = torch.arange(step.num_seqs, dtype=torch.int32, device=q.device)
+        table = (step.seq_start[:-1, None] + torch.arange(step.longest_run, dtype=torch.int32, device=q.device)[None, :]).contiguous()
+        local = dataclasses.replace(step, seq_slot=own)
+        return ragged_attention(qf, keys, values, s.scale, local, table, window=s.window)
 
 
 class MinGRU(nn.Module):

@@ -326,6 +326,40 @@ def test_whole_prompt_layers_and_logits(tmp_path_factory, name):
 
 
 @pytest.mark.parametrize("name", sorted(T.CONFIGS))
+def test_whole_prompts_take_the_expanded_form_and_agree_with_the_oracle_and_with_portions(tmp_path_factory, name, monkeypatch):
+    """Prompts of 64 tokens and more that start their sequences expand keys / values per head from the step's own latent rows
+    instead of reading them through the absorbed form: two unequal prompts in one step, and a long first portion followed by
+    portions and decoded tokens that read the same rows from the cache."""
+    from lite_llama_amd.executor.ragged import RaggedRunner
+    from lite_llama_amd.model_layers import LatentAttention
+    from oracle import rukedra as O
+
+    calls = []
+    plain = LatentAttention._expanded
+    monkeypatch.setattr(LatentAttention, "_expanded", lambda self, *a: (calls.append(1), plain(self, *a))[1])
+    model, cfg, tens, _ = _model(tmp_path_factory, name, torch.float32)
+    a, b = L.prompt(cfg, 150, seed=11), L.prompt(cfg, 67, seed=12)
+    wa, wb = O.forward(cfg, tens, a)[0], O.forward(cfg, tens, b)[0]
+    runner = RaggedRunner(model, 512, 3, block_size=16, device=DEV)
+    sa, sb = runner.admit(), runner.admit()
+    got = runner.step([(sa, a), (sb, b)], list(range(217)))
+    latent_layers = sum(1 for e in cfg["layers"] if e["type"] != "mingru")
+    assert len(calls) == latent_layers
+    _close(got[:150], wa, 2e-5)
+    _close(got[150:], wb, 2e-5)
+    runner.release([sa, sb])
+    _close(_feed(runner, runner.admit(), a, [70, 3, 40, 1]), wa, 2e-5)      # the first portion expanded, the rest absorbed
+    assert len(calls) == 2 * latent_layers
+    runner.check_errors()
+    half, _, _, _ = _model(tmp_path_factory, name, torch.bfloat16)
+    r16 = RaggedRunner(half, 512, 2, block_size=16, device=DEV)
+    whole = _feed(r16, r16.admit(), a, [150]).float().cpu()                   # expanded
+    parts = _feed(r16, r16.admit(), a, [50, 50, 50]).float().cpu()            # absorbed
+    err = lambda x, y: (x.to(F64) - y.to(F64)).pow(2).mean(-1).sqrt().median().item()   # noqa: E731
+    assert err(whole, wa) < 0.06 * wa.std().item() and err(parts, whole) < 0.04 * wa.std().item()
+
+
+@pytest.mark.parametrize("name", sorted(T.CONFIGS))
 @pytest.mark.parametrize("sizes", [[1], [2], [3, 2, 7, 1, 16, 5], [40, 1]])
 def test_portions_and_token_by_token_decoding_equal_the_whole_prompt(tmp_path_factory, name, sizes):
     """Portions down to two tokens, pure token-by-token decoding from the first token on, and a long portion followed by
