@@ -311,11 +311,12 @@ class DenseMLP(nn.Module):
 
 class LatentAttention(nn.Module):
     """Attention whose keys and values are up-projections of ONE cached latent row per token, plus a rotated key part that
-    all heads share.  Run in the absorbed form: the cache holds ``[latent | rotated key part]`` (one key/value head of key
-    width ``kv_rank + rot_dim``; the values are the first ``kv_rank`` columns of the same rows), a head's query becomes
+    all heads share.  The cache is read in the absorbed form: it holds ``[latent | rotated key part]`` (one key/value head of
+    key width ``kv_rank + rot_dim``; the values are the first ``kv_rank`` columns of the same rows), a head's query becomes
     ``[W_uk^T q_unrotated | rotate(q_rotated)]`` and its output ``W_uv (weights . latents)`` -- two batched products over the
-    heads around the attention kernel.  Everything that reads the mixer's input (query or query latent, key/value latent,
-    output gate, ``extra`` columns of the layer) is one projection."""
+    heads around the attention kernel.  Whole prompts (every sequence of the step at position 0) need nothing from the cache
+    and expand keys and values per head from the step's own rows instead (:meth:`_expanded`).  Everything that reads the
+    mixer's input (query or query latent, key/value latent, output gate, ``extra`` columns of the layer) is one projection."""
 
     def __init__(self, width: int, spec: MixerSpec, eps: float, extra: int = 0):
         super().__init__()
