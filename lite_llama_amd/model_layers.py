@@ -224,8 +224,9 @@ def _rukedra_geometry(config: Mapping, name: str) -> LayeredGeometry:
         else:
             raise ValueError(f"unsupported feed-forward kind {mlp.get('kind')!r}; supported: dense, moe")
         owner = entry.get("weights_of")
-        if owner is not None and not (0 <= int(owner) < index and config["layers"][int(owner)].get("weights_of") is None):
-            raise ValueError(f"layer {index} borrows the weights of layer {owner}, which is not an earlier layer with its own")
+        if owner is not None and not (0 <= int(owner) < len(config["layers"]) and int(owner) != index
+                                      and config["layers"][int(owner)].get("weights_of") is None):
+            raise ValueError(f"layer {index} borrows the weights of layer {owner}, which is not another layer with weights of its own")
         layers.append(LayerSpec(spec, ff=mspec.ff if mspec else 0, mlp_kind=mspec.kind if mspec else "dense", mlp=mspec,
                                 weights_of=None if owner is None else int(owner)))
     norm = config["norm"]
@@ -533,10 +534,9 @@ class LayeredLM(nn.Module):
         self.embed_tokens = nn.Embedding(geo.vocab_size, geo.width, dtype=torch.float16)
         self.embed_tokens.weight.requires_grad_(False)
         make = SandwichLayer if geo.sandwich else MixerLayer
-        built: list[nn.Module] = []
-        for spec in geo.layers:   # a layer that borrows weights IS the other layer's module; its cache run stays its own
-            built.append(built[spec.weights_of] if spec.weights_of is not None else make(geo, spec))
-        self.layers = nn.ModuleList(built)
+        # a layer that borrows weights IS the other layer's module (which may come later in the stack); its cache run stays its own
+        built = [make(geo, spec) if spec.weights_of is None else None for spec in geo.layers]
+        self.layers = nn.ModuleList(built[i] if spec.weights_of is None else built[spec.weights_of] for i, spec in enumerate(geo.layers))
         if geo.looped:
             self.loop_in = _linear(2 * geo.width, geo.width)
             self.loop_step = nn.Parameter(torch.zeros(geo.loop_times, geo.width, dtype=torch.float16), requires_grad=False)

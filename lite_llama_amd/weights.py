@@ -621,6 +621,10 @@ def _rukedra_translator(geo) -> Translator:
         return out
 
     members = [fused(spec) if spec.weights_of is None else {} for spec in geo.layers]
+    # a shared module is listed under the FIRST layer that uses it (a borrower in front of its owner gives the parameters its name)
+    listed: dict[int, int] = {}
+    for index, spec in enumerate(geo.layers):
+        listed.setdefault(index if spec.weights_of is None else spec.weights_of, index)
 
     def translate(key: str) -> Target:
         if key in fixed:
@@ -629,16 +633,17 @@ def _rukedra_translator(geo) -> Translator:
         if m is None or int(m.group(1)) >= len(geo.layers):
             return key, whole  # unknown: load_weights reports it
         index, leaf = int(m.group(1)), m.group(2)
+        at = listed.get(index, index)
         if leaf in members[index]:
             name, first, rows = members[index][leaf]
-            return f"layers.{index}.{name}", Region(rows=(first, rows))
+            return f"layers.{at}.{name}", Region(rows=(first, rows))
         e = expert_leaf.match(leaf)
         if e is not None:
             k, proj = int(e.group(1)), e.group(2)
             if proj == "down":
-                return f"layers.{index}.mlp.down_weight", expert(k)
-            return f"layers.{index}.mlp.gate_up_weight", expert_half(k, 0 if proj == "gate" else 1)
-        return f"layers.{index}.{plain.get(leaf, leaf)}", whole
+                return f"layers.{at}.mlp.down_weight", expert(k)
+            return f"layers.{at}.mlp.gate_up_weight", expert_half(k, 0 if proj == "gate" else 1)
+        return f"layers.{at}.{plain.get(leaf, leaf)}", whole
 
     return translate
 

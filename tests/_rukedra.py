@@ -66,6 +66,9 @@ CONFIGS = {
     # twenty heads on one latent (two column tiles of the grouped decode form), four norm groups, a window longer than a page
     "wide": config([latent2(20, 8, 8, 8, 24, mlp=dense(40)), latent(2, 8, 24, 16, 32, 16, 21, mlp=dense(40), original=512),
                     mingru(64, mlp=moe(8, 4, 8, groups=(2, 1), scale=2.5, shared=8))], width=64, vocab=71, groups=4, softcap=30.0),
+    # a layer that borrows from a LATER layer (the shared module is listed under the borrower), two norm groups, top 1 of 2
+    "fwd": config([borrowed(mingru(24, mlp=moe(2, 1, 16, shared=8)), 2), latent2(3, 8, 8, 16, 24, mlp=dense(40)),
+                   mingru(24, mlp=moe(2, 1, 16, shared=8)), latent(2, 16, 8, 8, 16, 8, 3)], width=48, vocab=59, groups=2),
 }
 
 

@@ -42,7 +42,7 @@ def test_reader_refuses_what_it_cannot_build(bad):
     elif bad == "groups":
         cfg["norm"]["groups"] = 5
     elif bad == "borrow":
-        cfg["layers"][3]["weights_of"] = 4
+        cfg["layers"][4]["weights_of"] = 3                          # layer 3 borrows itself: it owns nothing
     elif bad == "top":
         cfg["layers"][0]["mlp"]["router"]["groups"]["keep"] = 1     # one group of two experts cannot give three
     else:
@@ -81,7 +81,7 @@ def test_checkpoint_lands_in_the_fused_projections_and_borrowed_layers_share_mod
     for i, entry in enumerate(cfg["layers"]):
         layer, p = model.layers[i], f"l{entry.get('weights_of', i)}."
         if entry.get("weights_of") is not None:
-            assert layer is model.layers[entry["weights_of"]]
+            assert layer is model.layers[entry["weights_of"]]          # (the owner may come later in the stack)
             continue
         w = layer.mixer.in_proj.weight
         assert torch.equal(w[-W:], tens[p + "rg1"]) and torch.equal(layer.rg1_bias, tens[p + "rg1.b"])
@@ -110,7 +110,8 @@ def test_checkpoint_lands_in_the_fused_projections_and_borrowed_layers_share_mod
             assert torch.equal(layer.mlp.in_proj.weight[-W:], tens[p + "rg2"])
     # a missing and an unknown tensor are both named
     short = dict(tens)
-    del short["l0.rg1.b"]
+    owner = next(i for i, e in enumerate(cfg["layers"]) if e.get("weights_of") is None)
+    del short[f"l{owner}.rg1.b"]
     with pytest.raises(ValueError, match="rg1_bias"):
         load_pretrained(L.write(tmp_path / "short", cfg, short), device="cpu", dtype=torch.float32)
     with pytest.raises(ValueError, match="unknown parameter"):
